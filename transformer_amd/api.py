@@ -32,7 +32,10 @@ def open_model_source(path):
         rows = f.shape("token_embd.weight")[0] if "token_embd.weight" in f else None
         return arch, arch.config_from_gguf(f.metadata, rows), f
     arch, cfg = read_model_folder_config(p)
-    return arch, cfg, TensorFolder(p)
+    file = TensorFolder(p)
+    if arch.complete_config is not None:
+        cfg = arch.complete_config(cfg, file)
+    return arch, cfg, file
 
 
 def load_model(path, dtype=None, device="cuda:0", verbose=False) -> DecoderModel:

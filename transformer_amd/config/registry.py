@@ -14,7 +14,7 @@ from __future__ import annotations
 import json
 from dataclasses import dataclass
 from pathlib import Path
-from typing import Callable, Dict
+from typing import Callable, Dict, Optional
 
 from .spec import ConfigError
 
@@ -30,6 +30,9 @@ class Architecture:
     config_from_gguf: Callable      # (metadata dict, vocab rows) -> typed config, or None
     model_spec: Callable            # typed config -> ModelSpec
     weight_sources: Callable        # (typed config, ModelSpec, file format) -> {param: Source}
+    # (typed config, opened tensor file) -> typed config: for a size that only a tensor's
+    # shape gives; None where config.json says everything
+    complete_config: Optional[Callable] = None
 
 
 _ARCHITECTURES: Dict[str, Architecture] = {}
@@ -53,14 +56,16 @@ def get_architecture(name: str) -> Architecture:
 
 
 def architecture_of_config_json(d: dict) -> Architecture:
-    """config.json names its model class in ``architectures`` (first entry);
-    ``model_type`` is the fallback."""
+    """config.json names its model class in ``architectures`` (first entry) or in
+    ``architecture``; ``model_type`` is the fallback."""
     names = d.get("architectures")
     if isinstance(names, (list, tuple)) and names:
         return get_architecture(names[0])
+    if isinstance(d.get("architecture"), str):
+        return get_architecture(d["architecture"])
     if "model_type" in d:
         return get_architecture(d["model_type"])
-    raise ConfigError("config.json has neither 'architectures' nor 'model_type'")
+    raise ConfigError("config.json has none of 'architectures', 'architecture' and 'model_type'")
 
 
 def read_model_folder_config(folder):

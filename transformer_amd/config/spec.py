@@ -122,3 +122,116 @@ class ModelSpec:
                 if self.schedule[run.cache_of].cache_of is not None:
                     raise ConfigError(f"schedule[{i}].cache_of={run.cache_of} names an entry "
                                       f"that itself borrows a cache")
+
+
+# ---------------------------------------------------------------------------------------------
+# Parts beyond the Llama decoder's. Each is usable by any architecture: its sizes and constants
+# are fields, and the executor of its ``kind`` is registered in ``transformer_amd.parts``.
+
+@dataclass(frozen=True)
+class ScalarNormSpec:
+    """RMS norm whose gain is ONE number for all coordinates (the file holds a 0-d tensor)."""
+    size: int
+    eps: float
+    kind: str = "rmsnorm_scalar"
+
+
+@dataclass(frozen=True)
+class GLUSpec:
+    """down(act(gate(h)) * up(h)); activation "silu" or "gelu_tanh"."""
+    hidden: int
+    intermediate: int
+    activation: str = "silu"
+    bias: bool = False
+    kind: str = "glu"
+
+
+@dataclass(frozen=True)
+class PairHashEmbedSpec:
+    """Added to the embedded rows: row (previous token * mul_prev + token * mul_cur) mod
+    buckets of a second table, and row ``buckets`` (the last) for a sequence's first token."""
+    hidden: int
+    buckets: int
+    mul_prev: int
+    mul_cur: int
+    kind: str = "pair_hash_embed"
+
+
+@dataclass(frozen=True)
+class LogitScaleSpec:
+    """logits *= scale."""
+    scale: float
+    kind: str = "logit_scale"
+
+
+@dataclass(frozen=True)
+class NormedAttentionSpec:
+    """Causal grouped-query softmax attention whose keys and values have widths of their own.
+
+    qk_norm: q and k are RMS-normed over their whole projection (all heads at once) with a
+    weight per coordinate, before the rotation. rot_dims: the first coordinates of every head
+    that are rotated, in pairs (i, i + rot_dims/2), by position * rot_base^(-2i/rot_dims); 0 =
+    no rotation. value_mix: None; "source" = this mixer's values are kept for the step;
+    "mix" = v <- (1 - lambda) v + lambda * (the source's values of the same token), lambda a
+    learned number, and the mixed v is what the cache holds."""
+    hidden: int
+    num_heads: int
+    num_kv_heads: int
+    key_dim: int
+    value_dim: int
+    scale: float
+    eps: float
+    qk_norm: bool = True
+    rot_dims: int = 0
+    rot_base: float = 10000.0
+    value_mix: Optional[str] = None
+    window: Optional[int] = None
+    kind: str = "attention_normed"
+
+
+@dataclass(frozen=True)
+class DiagonalRecurrenceSpec:
+    """Two branches of ``channels``: y = gelu_tanh(Wy h + b) and u = causal conv of ``taps``
+    over (Wx h + b); gates r, i = sigmoid of block-diagonal maps of u (``blocks`` blocks);
+    a = exp(-decay_scale * r * softplus(lam)); S <- a S + sqrt(1 - a^2) * i * u; out = Wo (S * y).
+    State per sequence: S and the last taps - 1 inputs of the convolution."""
+    hidden: int
+    channels: int
+    blocks: int
+    taps: int
+    decay_scale: float = 8.0
+    kind: str = "diagonal_recurrence"
+
+
+@dataclass(frozen=True)
+class GatedLinearAttentionSpec:
+    """Per head a matrix state S [key_dim, value_dim]: S <- diag(alpha) S + k v^T, o = S^T q,
+    q scaled by key_dim^-1/2, alpha = sigmoid(W2 (W1 h) + b)^(1/tau) per key channel (W1 maps
+    to ``rank`` numbers); o is RMS-normed per head, gated by silu(Wg h) and projected."""
+    hidden: int
+    num_heads: int
+    key_dim: int
+    value_dim: int
+    rank: int
+    tau: float
+    eps: float
+    kind: str = "gated_linear_attention"
+
+
+@dataclass(frozen=True)
+class GatedBlockSpec:
+    """x += mult * gate1 * mixer(shift(norm1(x))); x += mult * gate2 * ffn(norm2(x)).
+
+    gated: each sublayer's result is multiplied by sigmoid(W h + b), h the normed input of the
+    sublayer (before the shift). token_shift: the mixer reads h_t + (h_{t-1} - h_t) * mu with
+    a learned mu per coordinate; h_{t-1} is the unshifted row of the previous token (zeros
+    before the first) and is carried between steps. ffn None: the block has one sublayer."""
+    norm1: object
+    mixer: object
+    norm2: object = None
+    ffn: object = None
+    hidden: int = 0
+    mult: float = 1.0
+    gated: bool = True
+    token_shift: bool = True
+    kind: str = "gated_prenorm"

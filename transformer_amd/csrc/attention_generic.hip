@@ -1,6 +1,6 @@
 // Causal grouped-query attention over the paged cache, float32 arithmetic on the
-// vector ALU, for any head size that is a multiple of 16 up to 256 and both
-// storage types. It serves prompts and single tokens alike.
+// vector ALU, for any key width and any value width up to 256 (the two may differ)
+// and both storage types. It serves prompts and single tokens alike.
 //
 // A workgroup owns 16 "rows" of one (sequence, kv head): row = (query token,
 // query head inside the kv head's group), so the heads of a group share every
@@ -29,7 +29,7 @@ __global__ __launch_bounds__(256) void attn_generic_kernel(
     const T* __restrict__ q, int q_stride, T* __restrict__ out, int out_stride,
     const T* __restrict__ kcache, const T* __restrict__ vcache,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ cu_q,
-    const int* __restrict__ pos0, int nh, int nkv, int dh, float scale, int window) {
+    const int* __restrict__ pos0, int nh, int nkv, int dh, int dv, float scale, int window) {
   extern __shared__ float smem[];
   const int group = nh / nkv;
   const int b = blockIdx.z, kvh = blockIdx.y;
@@ -43,7 +43,7 @@ __global__ __launch_bounds__(256) void attn_generic_kernel(
   const bool row_ok = row < nrows;
   const int qi = row_ok ? row / group : 0;
   const int head = kvh * group + (row_ok ? row % group : 0);
-  const int DHP = dh + 1;
+  const int DHP = (dh > dv ? dh : dv) + 1;
   float* Qs = smem;                 // [ROWS][dh]
   float* KVs = Qs + ROWS * dh;      // [CHUNK][dh + 1]
   float* Ps = KVs + CHUNK * DHP;    // [ROWS][CHUNK]
@@ -72,7 +72,7 @@ __global__ __launch_bounds__(256) void attn_generic_kernel(
     if (my_start < 0) my_start = 0;
   }
 
-  const int nd = dh / 16;
+  const int nd = (dv + 15) / 16;          // output columns lane, lane + 16, ... of this lane
   float acc[16];
 #pragma unroll
   for (int i = 0; i < 16; ++i) acc[i] = 0.f;
@@ -83,7 +83,7 @@ __global__ __launch_bounds__(256) void attn_generic_kernel(
     const int key0 = c * CHUNK;
     const size_t page = (size_t)table[key0 / TA_PAGE];
     const size_t base = ((page * nkv + kvh) * TA_PAGE + key0 % TA_PAGE) * (size_t)dh;
-    const size_t vbase = (page * nkv + kvh) * (size_t)dh * TA_PAGE + key0 % TA_PAGE;
+    const size_t vbase = (page * nkv + kvh) * (size_t)dv * TA_PAGE + key0 % TA_PAGE;
     // ---- K chunk -> LDS (keys that are not written yet read as zero)
     for (int i = threadIdx.x; i < CHUNK * dh; i += 256) {
       const int k = i / dh, d = i - k * dh;
@@ -121,7 +121,7 @@ __global__ __launch_bounds__(256) void attn_generic_kernel(
     Ps[rloc * CHUNK + lane + 16] = e1;
     __syncthreads();
     // ---- V chunk -> LDS
-    for (int i = threadIdx.x; i < CHUNK * dh; i += 256) {     // value pages are [dh][TA_PAGE]
+    for (int i = threadIdx.x; i < CHUNK * dv; i += 256) {     // value pages are [dv][TA_PAGE]
       const int d = i / CHUNK, k = i - d * CHUNK;
       KVs[k * DHP + d] = (key0 + k < tile_end) ? to_f32(vcache[vbase + (size_t)d * TA_PAGE + k]) : 0.f;
     }
@@ -133,51 +133,70 @@ __global__ __launch_bounds__(256) void attn_generic_kernel(
         const float* vr = KVs + k * DHP + lane;
 #pragma unroll
         for (int i = 0; i < 16; ++i)
-          if (i < nd) acc[i] = fmaf(p, vr[16 * i], acc[i]);
+          if (i < nd && 16 * i + lane < dv) acc[i] = fmaf(p, vr[16 * i], acc[i]);
       }
     }
     __syncthreads();
   }
   if (row_ok) {
     const float inv = l > 0.f ? 1.0f / l : 0.f;
-    T* o = out + (size_t)(q0 + qi) * out_stride + (size_t)head * dh + lane;
+    T* o = out + (size_t)(q0 + qi) * out_stride + (size_t)head * dv + lane;
 #pragma unroll
     for (int i = 0; i < 16; ++i)
-      if (i < nd) o[16 * i] = from_f32<T>(acc[i] * inv);
+      if (i < nd && 16 * i + lane < dv) o[16 * i] = from_f32<T>(acc[i] * inv);
   }
 }
 
 // q: [nt, ...] with q_stride elements between tokens, head h at offset h*dh.
-// out: [nt, nh*dh] with out_stride elements between tokens.
-// kcache: one layer, [pages][nkv][TA_PAGE][dh]; vcache: [pages][nkv][dh][TA_PAGE].
+// out: [nt, nh*dv] with out_stride elements between tokens.
+// kcache: one layer, [pages][nkv][TA_PAGE][dh]; vcache: [pages][nkv][dv][TA_PAGE].
 // block_table: [B][max_blocks].
 // cu_q: [B+1] first token of each sequence in q. pos0: [B] tokens cached before this
 // step (the step's own keys are already in the cache). window <= 0: all keys.
-extern "C" int ta_attention_generic(hipStream_t stream, int dtype, const void* q, int q_stride,
+static int attention_generic_launch(hipStream_t stream, int dtype, const void* q, int q_stride,
                                     void* out, int out_stride, const void* kcache,
                                     const void* vcache, const int* block_table, int max_blocks,
                                     const int* cu_q, const int* pos0, int batch, int max_qlen,
-                                    int nh, int nkv, int dh, float scale, int window) {
+                                    int nh, int nkv, int dh, int dv, float scale, int window) {
   TA_REQUIRE(batch >= 0 && max_qlen >= 0, "ta_attention_generic: bad batch=%d max_qlen=%d", batch, max_qlen);
   TA_REQUIRE(nh > 0 && nkv > 0 && nh % nkv == 0, "ta_attention_generic: %d heads do not divide into %d kv heads", nh, nkv);
-  TA_REQUIRE(dh >= 16 && dh <= 256 && dh % 16 == 0,
-             "ta_attention_generic: head size %d is not a multiple of 16 in [16, 256]", dh);
-  TA_REQUIRE(q_stride >= nh * dh && out_stride >= nh * dh, "ta_attention_generic: strides too small");
+  TA_REQUIRE(dh >= 1 && dh <= 256 && dv >= 1 && dv <= 256,
+             "ta_attention_generic: key width %d / value width %d outside [1, 256]", dh, dv);
+  TA_REQUIRE(q_stride >= nh * dh && out_stride >= nh * dv, "ta_attention_generic: strides too small");
   TA_REQUIRE(max_blocks > 0, "ta_attention_generic: empty block table");
   TA_REQUIRE(batch <= 65535 && nkv <= 65535, "ta_attention_generic: grid too large");
   if (batch == 0 || max_qlen == 0) return 0;
   const int group = nh / nkv;
   dim3 g((max_qlen * group + ROWS - 1) / ROWS, nkv, batch), blk(256);
-  const size_t lds = (size_t)(ROWS * dh + CHUNK * (dh + 1) + ROWS * CHUNK) * sizeof(float);
+  const size_t lds = (size_t)(ROWS * dh + CHUNK * ((dh > dv ? dh : dv) + 1) + ROWS * CHUNK) * sizeof(float);
   if (dtype == TA_F32)
     attn_generic_kernel<float><<<g, blk, lds, stream>>>(
         (const float*)q, q_stride, (float*)out, out_stride, (const float*)kcache,
-        (const float*)vcache, block_table, max_blocks, cu_q, pos0, nh, nkv, dh, scale, window);
+        (const float*)vcache, block_table, max_blocks, cu_q, pos0, nh, nkv, dh, dv, scale, window);
   else if (dtype == TA_BF16)
     attn_generic_kernel<bf16_t><<<g, blk, lds, stream>>>(
         (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kcache,
-        (const bf16_t*)vcache, block_table, max_blocks, cu_q, pos0, nh, nkv, dh, scale, window);
+        (const bf16_t*)vcache, block_table, max_blocks, cu_q, pos0, nh, nkv, dh, dv, scale, window);
   else
     return ta_fail("ta_attention_generic: unknown dtype %d", dtype);
   return ta_check_launch("ta_attention_generic");
+}
+
+extern "C" int ta_attention_generic(hipStream_t stream, int dtype, const void* q, int q_stride,
+                                    void* out, int out_stride, const void* kcache,
+                                    const void* vcache, const int* block_table, int max_blocks,
+                                    const int* cu_q, const int* pos0, int batch, int max_qlen,
+                                    int nh, int nkv, int dh, float scale, int window) {
+  return attention_generic_launch(stream, dtype, q, q_stride, out, out_stride, kcache, vcache, block_table,
+                                  max_blocks, cu_q, pos0, batch, max_qlen, nh, nkv, dh, dh, scale, window);
+}
+
+// The same with values of another width than the keys: dv columns per head in vcache and out.
+extern "C" int ta_attention_generic_dv(hipStream_t stream, int dtype, const void* q, int q_stride,
+                                       void* out, int out_stride, const void* kcache,
+                                       const void* vcache, const int* block_table, int max_blocks,
+                                       const int* cu_q, const int* pos0, int batch, int max_qlen,
+                                       int nh, int nkv, int dh, int dv, float scale, int window) {
+  return attention_generic_launch(stream, dtype, q, q_stride, out, out_stride, kcache, vcache, block_table,
+                                  max_blocks, cu_q, pos0, batch, max_qlen, nh, nkv, dh, dv, scale, window);
 }

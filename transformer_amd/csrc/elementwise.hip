@@ -523,7 +523,13 @@ extern "C" int ta_rope_kv_write(hipStream_t stream, int dtype, void* qkv, const 
 // ------------------------------------------------------------------ SwiGLU
 // out[t, i] = silu(g) * u, g = gu[t, i] (+bias[i]), u = gu[t, di + i] (+bias[di + i]),
 // silu(z) = z / (1 + exp(-z)), all in float32, rounded once. grid (chunks of a row, rows).
-template <typename T>
+// act 0: silu(a) = a / (1 + exp(-a)); act 1: the tanh form of gelu
+template <int ACT> __device__ __forceinline__ float glu_act(float a) {
+  if (ACT == 0) return a / (1.0f + expf(-a));
+  return 0.5f * a * (1.0f + tanhf(0.7978845608028654f * (a + 0.044715f * a * a * a)));
+}
+
+template <typename T, int ACT>
 __global__ void swiglu_kernel(const T* __restrict__ gu, const float* __restrict__ bias,
                               T* __restrict__ out, int di) {
   const size_t t = blockIdx.y;
@@ -544,7 +550,7 @@ __global__ void swiglu_kernel(const T* __restrict__ gu, const float* __restrict_
         a += bias[4 * c + e];
         u += bias[di + 4 * c + e];
       }
-      r[e] = a / (1.0f + expf(-a)) * u;
+      r[e] = glu_act<ACT>(a) * u;
     }
     ov.set(r[0], r[1], r[2], r[3]);
     ov.store(o + 4 * c);
@@ -555,29 +561,40 @@ __global__ void swiglu_kernel(const T* __restrict__ gu, const float* __restrict_
         a += bias[i];
         u += bias[di + i];
       }
-      o[i] = from_f32<T>(a / (1.0f + expf(-a)) * u);
+      o[i] = from_f32<T>(glu_act<ACT>(a) * u);
     }
   }
 }
 
-extern "C" int ta_swiglu(hipStream_t stream, int dtype, const void* gate_up, const float* bias,
-                         void* out, int nt, int di) {
-  TA_REQUIRE(nt >= 0 && di > 0, "ta_swiglu: bad sizes nt=%d di=%d", nt, di);
-  TA_REQUIRE(nt <= 65535 * 64, "ta_swiglu: too many rows for one launch");
+// out = act(gate) * up over rows of [gate | up]; act 0 = silu, 1 = gelu (tanh form).
+extern "C" int ta_glu(hipStream_t stream, int dtype, int act, const void* gate_up, const float* bias,
+                      void* out, int nt, int di) {
+  TA_REQUIRE(nt >= 0 && di > 0, "ta_glu: bad sizes nt=%d di=%d", nt, di);
+  TA_REQUIRE(nt <= 65535 * 64, "ta_glu: too many rows for one launch");
+  TA_REQUIRE(act == 0 || act == 1, "ta_glu: unknown activation %d", act);
   if (nt == 0) return 0;
   const int per_block = 256 * 4;
   for (int t0 = 0; t0 < nt; t0 += 65535) {
     const int rows = nt - t0 < 65535 ? nt - t0 : 65535;
     dim3 g((di + per_block - 1) / per_block, rows), b(256);
     const size_t in_off = (size_t)t0 * 2 * di, out_off = (size_t)t0 * di;
-    if (dtype == TA_F32)
-      swiglu_kernel<float><<<g, b, 0, stream>>>((const float*)gate_up + in_off, bias, (float*)out + out_off, di);
+    if (dtype == TA_F32 && act == 0)
+      swiglu_kernel<float, 0><<<g, b, 0, stream>>>((const float*)gate_up + in_off, bias, (float*)out + out_off, di);
+    else if (dtype == TA_F32)
+      swiglu_kernel<float, 1><<<g, b, 0, stream>>>((const float*)gate_up + in_off, bias, (float*)out + out_off, di);
+    else if (dtype == TA_BF16 && act == 0)
+      swiglu_kernel<bf16_t, 0><<<g, b, 0, stream>>>((const bf16_t*)gate_up + in_off, bias, (bf16_t*)out + out_off, di);
     else if (dtype == TA_BF16)
-      swiglu_kernel<bf16_t><<<g, b, 0, stream>>>((const bf16_t*)gate_up + in_off, bias, (bf16_t*)out + out_off, di);
+      swiglu_kernel<bf16_t, 1><<<g, b, 0, stream>>>((const bf16_t*)gate_up + in_off, bias, (bf16_t*)out + out_off, di);
     else
-      return ta_fail("ta_swiglu: unknown dtype %d", dtype);
+      return ta_fail("ta_glu: unknown dtype %d", dtype);
   }
-  return ta_check_launch("ta_swiglu");
+  return ta_check_launch("ta_glu");
+}
+
+extern "C" int ta_swiglu(hipStream_t stream, int dtype, const void* gate_up, const float* bias,
+                         void* out, int nt, int di) {
+  return ta_glu(stream, dtype, 0, gate_up, bias, out, nt, di);
 }
 
 // ------------------------------------------------------------------ random fill

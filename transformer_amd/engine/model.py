@@ -88,6 +88,20 @@ class DecoderModel:
                     raise ValueError(f"schedule[{i}] borrows the cache of entry {run.cache_of}, "
                                      f"whose layout differs")
                 self.cache_layer.append(self.cache_layer[run.cache_of])
+        # a part around the blocks (after the embedding, on the logits) that keeps something per
+        # sequence names its need as a mixer does and gets cache layers behind the blocks'
+        self.extra_layer: Dict[str, object] = {}
+        for name, part in self._extras().items():
+            need = getattr(part, "cache_need", lambda: None)()
+            if need is None:
+                continue
+            several = isinstance(need, (list, tuple))
+            layers = []
+            for one in (need if several else [need]):
+                layers.append(len(self.cache_needs))
+                self.cache_needs.append(one)
+                self.cache_planners.append(None)
+            self.extra_layer[name] = tuple(layers) if several else layers[0]
         self.w: Dict[str, torch.Tensor] = {}
         self.ws = Workspace(self.device)
         self.uploader = Uploader(self.device)
@@ -173,7 +187,7 @@ class DecoderModel:
             x = kernels.embed(self.w["embed"], ctx.tokens,
                               self.ws.take("model.x", (ctx.nt, s.hidden), torch.float32))
             if self.after_embed is not None:
-                self.after_embed.run(x, ctx)
+                self._run_extra("after_embed", x, ctx, cache)
         if self.dump is not None:
             self.dump("embed", x)
         pending = (None, None)
@@ -196,10 +210,17 @@ class DecoderModel:
             with span(ctx, "head"):
                 linear(hn, self.w["head"], logits)
                 if self.on_logits is not None:
-                    self.on_logits.run(logits, ctx)
+                    self._run_extra("on_logits", logits, ctx, cache)
         if self.dump is not None:
             self.dump("logits", logits)
         return logits
+
+    def _run_extra(self, name, t, ctx, cache):
+        part = getattr(self, name)
+        if name in self.extra_layer:
+            part.run(t, ctx, cache, self.extra_layer[name])
+        else:
+            part.run(t, ctx)
 
     @staticmethod
     def _stream_with(x, pending) -> torch.Tensor:
@@ -208,6 +229,8 @@ class DecoderModel:
         if isinstance(pending, kernels.RowScale):
             return x.clone()                      # the block's last product has added itself
         delta, bias = pending
+        if isinstance(delta, kernels.GatedDelta):
+            return delta.applied(x)
         full = x.clone()
         if delta is not None:
             full += delta.float().sum(0) if delta.dim() == 3 else delta.float()

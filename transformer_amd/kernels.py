@@ -85,10 +85,11 @@ def _rows2d(t: torch.Tensor, name: str):
     return t.shape[0], t.stride(0)
 
 
-def _check_cache_layer(what, kcache, vcache, num_kv_heads, head_dim):
-    """keys [pages, nkv, PAGE, dh]; values transposed inside a page: [pages, nkv, dh, PAGE]."""
+def _check_cache_layer(what, kcache, vcache, num_kv_heads, head_dim, value_dim=None):
+    """keys [pages, nkv, PAGE, dh]; values transposed inside a page: [pages, nkv, dv, PAGE]
+    (dv = dh unless a value width is named)."""
     wk = (kcache.shape[0], num_kv_heads, PAGE, head_dim)
-    wv = (kcache.shape[0], num_kv_heads, head_dim, PAGE)
+    wv = (kcache.shape[0], num_kv_heads, head_dim if value_dim is None else value_dim, PAGE)
     if tuple(kcache.shape) != wk or tuple(vcache.shape) != wv:
         raise KernelError(f"{what}: cache layer is {tuple(kcache.shape)} / {tuple(vcache.shape)}, "
                           f"expected {wk} / {wv}")
@@ -806,3 +807,319 @@ def convert(src: torch.Tensor, dst: torch.Tensor) -> torch.Tensor:
     _check(library().ta_convert(_stream(), c_int(_CONVERT_SRC[src.dtype]), c_int(_code(dst.dtype)),
                                 _ptr(src), _ptr(dst), c_longlong(src.numel())))
     return dst
+
+
+# ------------------------------------------------------------------ gated activations
+_GLU_ACTS = {"silu": 0, "gelu_tanh": 1}
+
+
+def glu(gate_up: torch.Tensor, out: torch.Tensor, activation: str = "silu",
+        bias: Optional[torch.Tensor] = None):
+    """out = act(gate_up[:, :di]) * gate_up[:, di:]; act "silu" or "gelu_tanh"."""
+    if activation not in _GLU_ACTS:
+        raise KernelError(f"glu: unknown activation {activation!r}; known: {sorted(_GLU_ACTS)}")
+    _dev(gate_up, "gate_up"); _dev(out, "out", gate_up.dtype)
+    nt, w = gate_up.shape
+    if w % 2 or out.shape != (nt, w // 2):
+        raise KernelError(f"glu: gate_up {tuple(gate_up.shape)} / out {tuple(out.shape)}")
+    if bias is not None:
+        _dev(bias, "bias", torch.float32)
+        if bias.numel() != w:
+            raise KernelError("glu: bias must hold one entry per gate_up column")
+    _check(library().ta_glu(_stream(), c_int(_code(gate_up.dtype)), c_int(_GLU_ACTS[activation]),
+                            _ptr(gate_up), _ptr(bias), _ptr(out), c_int(nt), c_int(w // 2)))
+    return out
+
+
+# ------------------------------------------------------------------ gated residual, token shift
+class GatedDelta:
+    """What a gated sublayer leaves for the next norm to add to the float32 residual stream:
+    x += mult * sigmoid(gate + gate_bias) * (delta + delta_bias). ``delta`` [nt, d] float32 (or
+    [planes, nt, d], added in order); ``gate`` [nt, d] float32, the gate's pre-activation, or
+    None for no gate."""
+
+    def __init__(self, delta, delta_bias=None, gate=None, gate_bias=None, mult: float = 1.0):
+        self.delta, self.delta_bias = delta, delta_bias
+        self.gate, self.gate_bias, self.mult = gate, gate_bias, float(mult)
+
+    def applied(self, x: torch.Tensor) -> torch.Tensor:
+        """x + this delta as a new tensor (debugging: the engine lets the next norm add it)."""
+        d = self.delta.float().sum(0) if self.delta.dim() == 3 else self.delta.float()
+        if self.delta_bias is not None:
+            d = d + self.delta_bias
+        if self.gate is not None:
+            g = self.gate if self.gate_bias is None else self.gate + self.gate_bias
+            d = d * torch.sigmoid(g)
+        return x + self.mult * d
+
+
+def gated_add_rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor,
+                      pending: Optional[GatedDelta] = None,
+                      rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """v = x[r] + pending (see ``GatedDelta``); out[i] = v / sqrt(mean(v^2) + eps) * weight.
+    Without ``rows`` v is stored back into x; with ``rows`` (int32) only those rows are
+    normalised and x is left as it is."""
+    _dev(x, "x", torch.float32); _dev(weight, "weight", torch.float32); _dev(out, "out")
+    nt, d = x.shape
+    if weight.shape != (d,):
+        raise KernelError(f"gated_add_rmsnorm: weight is {tuple(weight.shape)}, expected {(d,)}")
+    n_out = nt
+    if rows is not None:
+        _dev(rows, "rows", torch.int32)
+        n_out = rows.numel()
+    if out.shape != (n_out, d):
+        raise KernelError(f"gated_add_rmsnorm: out is {tuple(out.shape)}, expected {(n_out, d)}")
+    delta = dbias = gate = gbias = None
+    planes, plane, mult = 1, 0, 1.0
+    if pending is not None:
+        delta, dbias, gate, gbias, mult = (pending.delta, pending.delta_bias, pending.gate,
+                                           pending.gate_bias, pending.mult)
+        _dev(delta, "delta", torch.float32)
+        if delta.dim() == 3 and delta.shape[1:] == x.shape:
+            planes, plane = delta.shape[0], nt * d
+        elif delta.shape != x.shape:
+            raise KernelError(f"gated_add_rmsnorm: delta is {tuple(delta.shape)}, x {tuple(x.shape)}")
+        for t, n in ((dbias, "delta_bias"), (gbias, "gate_bias")):
+            if t is not None:
+                _dev(t, n, torch.float32)
+                if t.shape != (d,):
+                    raise KernelError(f"gated_add_rmsnorm: {n} must have one entry per column")
+        if gate is not None:
+            _dev(gate, "gate", torch.float32)
+            if gate.shape != x.shape:
+                raise KernelError(f"gated_add_rmsnorm: gate is {tuple(gate.shape)}, x {tuple(x.shape)}")
+    _check(library().ta_gated_add_rmsnorm(
+        _stream(), c_int(_code(out.dtype)), _ptr(x), _ptr(delta), c_int(planes), c_longlong(plane),
+        _ptr(dbias), _ptr(gate), _ptr(gbias), c_float(mult), _ptr(weight), _ptr(rows), _ptr(out),
+        c_int(n_out), c_int(d), c_float(eps), c_int(int(rows is None))))
+    return out
+
+
+def _step_tables(cu_q, slots, nt, what):
+    _dev(cu_q, "cu_q", torch.int32); _dev(slots, "slots", torch.int32)
+    batch = slots.numel()
+    if cu_q.numel() != batch + 1 or batch < 1 or nt < batch:
+        raise KernelError(f"{what}: cu_q / slots disagree about the batch ({cu_q.numel()} / {batch}, "
+                          f"{nt} tokens)")
+    return batch
+
+
+def token_shift(h: torch.Tensor, out: torch.Tensor, mu: torch.Tensor, state: torch.Tensor,
+                cu_q: torch.Tensor, slots: torch.Tensor) -> torch.Tensor:
+    """out[t] = h[t] + (h[t-1] - h[t]) * mu inside each sequence; the row before a sequence's
+    first token of the step comes from ``state`` [slots, d] (float32), which then takes the
+    sequence's last row of h."""
+    _dev(h, "h"); _dev(out, "out", h.dtype); _dev(mu, "mu", torch.float32)
+    _dev(state, "state", torch.float32)
+    nt, d = h.shape
+    batch = _step_tables(cu_q, slots, nt, "token_shift")
+    if out.shape != h.shape or mu.shape != (d,) or state.dim() != 2 or state.shape[1] != d:
+        raise KernelError(f"token_shift: h {tuple(h.shape)} out {tuple(out.shape)} mu {tuple(mu.shape)} "
+                          f"state {tuple(state.shape)}")
+    _check(library().ta_token_shift(_stream(), c_int(_code(h.dtype)), _ptr(h), _ptr(out), _ptr(mu),
+                                    _ptr(state), _ptr(cu_q), _ptr(slots), c_int(batch), c_int(nt), c_int(d)))
+    return out
+
+
+def pair_embed_add(x: torch.Tensor, table: torch.Tensor, tokens: torch.Tensor, last_token: torch.Tensor,
+                   cu_q: torch.Tensor, pos0: torch.Tensor, slots: torch.Tensor, buckets: int,
+                   mul_prev: int, mul_cur: int) -> torch.Tensor:
+    """x[t] += table[(previous token * mul_prev + token * mul_cur) % buckets], and
+    table[buckets] for a sequence's first token. ``last_token`` [slots] int32 holds every
+    sequence's last token between steps."""
+    _dev(x, "x", torch.float32); _dev(table, "table"); _dev(tokens, "tokens", torch.int32)
+    _dev(last_token, "last_token", torch.int32); _dev(pos0, "pos0", torch.int32)
+    nt, d = x.shape
+    batch = _step_tables(cu_q, slots, nt, "pair_embed_add")
+    if table.shape != (buckets + 1, d) or tokens.numel() != nt or pos0.numel() != batch:
+        raise KernelError(f"pair_embed_add: table {tuple(table.shape)} for {buckets} buckets of {d}, "
+                          f"{tokens.numel()} tokens for {nt} rows")
+    _check(library().ta_pair_embed_add(_stream(), c_int(_code(table.dtype)), _ptr(x), _ptr(table),
+                                       _ptr(tokens), _ptr(last_token), _ptr(cu_q), _ptr(pos0), _ptr(slots),
+                                       c_int(batch), c_int(nt), c_int(d), c_int(buckets),
+                                       c_longlong(mul_prev), c_longlong(mul_cur)))
+    return x
+
+
+def scale_(t: torch.Tensor, s: float) -> torch.Tensor:
+    """t *= s in place (float32)."""
+    _dev(t, "t", torch.float32)
+    _check(library().ta_scale_f32(_stream(), _ptr(t), c_longlong(t.numel()), c_float(s)))
+    return t
+
+
+# ------------------------------------------------------------------ attention with a value width of its own
+def qk_prepare(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, key_dim: int, value_dim: int,
+               eps: float, q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor],
+               angles: Optional[torch.Tensor], rot: int, mix: Optional[torch.Tensor] = None,
+               v_first: Optional[torch.Tensor] = None, v_keep: Optional[torch.Tensor] = None,
+               dest: Optional[torch.Tensor] = None, kcache: Optional[torch.Tensor] = None,
+               vcache: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """On rows [q | k | v] of ``qkv`` (nh*dk, nkv*dk, nkv*dv columns): RMS norm of q and of k
+    over all their heads at once (weights given: else none), rotation of the first ``rot``
+    coordinates of every head by ``angles`` [nt, rot/2, 2], v <- (1 - mix) v + mix v_first,
+    q written back in place, k and v stored at ``dest`` into the cache layer. ``v_keep``
+    receives the values before mixing."""
+    _dev(qkv, "qkv", contiguous=False)
+    nt, stride = _rows2d(qkv, "qkv")
+    nq, nk, nv = num_heads * key_dim, num_kv_heads * key_dim, num_kv_heads * value_dim
+    if qkv.shape[1] != nq + nk + nv:
+        raise KernelError(f"qk_prepare: rows of {qkv.shape[1]}, expected {nq + nk + nv}")
+    normed = q_weight is not None
+    if normed:
+        _dev(q_weight, "q_weight", torch.float32); _dev(k_weight, "k_weight", torch.float32)
+        if q_weight.shape != (nq,) or k_weight.shape != (nk,):
+            raise KernelError("qk_prepare: norm weights must cover the whole q and k projections")
+    if rot:
+        _dev(angles, "angles", torch.float32)
+        if tuple(angles.shape) != (nt, rot // 2, 2):
+            raise KernelError(f"qk_prepare: angles are {tuple(angles.shape)}, expected {(nt, rot // 2, 2)}")
+    else:
+        angles = None
+    if (mix is None) != (v_first is None):
+        raise KernelError("qk_prepare: mix and v_first go together")
+    if mix is not None:
+        _dev(mix, "mix", torch.float32); _dev(v_first, "v_first", qkv.dtype)
+        if mix.numel() != 1 or v_first.shape != (nt, nv):
+            raise KernelError(f"qk_prepare: mix {tuple(mix.shape)} / v_first {tuple(v_first.shape)}")
+    if v_keep is not None:
+        _dev(v_keep, "v_keep", qkv.dtype)
+        if v_keep.shape != (nt, nv):
+            raise KernelError(f"qk_prepare: v_keep is {tuple(v_keep.shape)}, expected {(nt, nv)}")
+    if dest is not None:
+        _dev(dest, "dest", torch.int32); _dev(kcache, "kcache", qkv.dtype); _dev(vcache, "vcache", qkv.dtype)
+        _check_cache_layer("qk_prepare", kcache, vcache, num_kv_heads, key_dim, value_dim)
+        if dest.numel() != nt:
+            raise KernelError("qk_prepare: dest must hold one entry per token")
+    _check(library().ta_qk_prepare(
+        _stream(), c_int(_code(qkv.dtype)), _ptr(qkv), c_int(stride), _ptr(q_weight), _ptr(k_weight),
+        c_float(eps), c_int(int(normed)), _ptr(angles), c_int(rot), _ptr(mix), _ptr(v_first), _ptr(v_keep),
+        _ptr(dest), _ptr(kcache if dest is not None else None), _ptr(vcache if dest is not None else None),
+        c_int(nt), c_int(num_heads), c_int(num_kv_heads), c_int(key_dim), c_int(value_dim)))
+    return qkv
+
+
+def attention_generic_dv(q, out, kcache, vcache, block_table, cu_q, pos0, max_qlen, num_heads,
+                         num_kv_heads, key_dim, value_dim, scale, window=None):
+    """``attention_generic`` for values of another width than the keys: q [nt, >= nh*dk],
+    out [nt, nh*dv], kcache [pages, nkv, PAGE, dk], vcache [pages, nkv, dv, PAGE]."""
+    _dev(q, "q", contiguous=False); _dev(out, "out", q.dtype, contiguous=False)
+    nt, qs = _rows2d(q, "q")
+    nto, os_ = _rows2d(out, "out")
+    if nt != nto or q.shape[1] < num_heads * key_dim or out.shape[1] != num_heads * value_dim:
+        raise KernelError(f"attention: q {tuple(q.shape)} / out {tuple(out.shape)} do not fit "
+                          f"{num_heads} heads of {key_dim} / {value_dim}")
+    _dev(kcache, "kcache", q.dtype); _dev(vcache, "vcache", q.dtype)
+    _check_cache_layer("attention", kcache, vcache, num_kv_heads, key_dim, value_dim)
+    _dev(block_table, "block_table", torch.int32); _dev(cu_q, "cu_q", torch.int32)
+    _dev(pos0, "pos0", torch.int32)
+    B = pos0.numel()
+    if cu_q.numel() != B + 1 or block_table.dim() != 2 or block_table.shape[0] != B:
+        raise KernelError("attention: cu_q / pos0 / block_table disagree about the batch size")
+    _check(library().ta_attention_generic_dv(
+        _stream(), c_int(_code(q.dtype)), _ptr(q), c_int(qs), _ptr(out), c_int(os_), _ptr(kcache),
+        _ptr(vcache), _ptr(block_table), c_int(block_table.shape[1]), _ptr(cu_q), _ptr(pos0),
+        c_int(B), c_int(max_qlen), c_int(num_heads), c_int(num_kv_heads), c_int(key_dim),
+        c_int(value_dim), c_float(scale), c_int(window or 0)))
+    return out
+
+
+# ------------------------------------------------------------------ recurrent mixers
+def _wcode(w: torch.Tensor, act: torch.dtype, what: str) -> int:
+    if w.dtype == act or (act == torch.bfloat16 and w.dtype == torch.float32):
+        return _code(w.dtype)
+    raise KernelError(f"{what}: activations are {act}, weights {w.dtype}")
+
+
+def rglru_gates(yx: torch.Tensor, channels: int, x_bias, taps, conv_bias, conv_state, gates_w, gates_b,
+                lam, decay_scale: float, cu_q, slots, a_out: torch.Tensor, b_out: torch.Tensor):
+    """Decay a_t and input term of the gated diagonal recurrence for every token of the step.
+    yx [nt, 2C]: the y branch, then the x branch (before their biases). taps [C, K], conv_state
+    [slots, K-1, C]; gates_w [2*blocks, bs, bs] (recurrence-gate blocks, then input-gate blocks),
+    gates_b [2*blocks, bs]; a_out, b_out [nt, C] float32."""
+    _dev(yx, "yx", contiguous=False)
+    nt, stride = _rows2d(yx, "yx")
+    C = channels
+    batch = _step_tables(cu_q, slots, nt, "rglru_gates")
+    for t, n in ((x_bias, "x_bias"), (taps, "taps"), (conv_bias, "conv_bias"), (conv_state, "conv_state"),
+                 (gates_b, "gates_b"), (lam, "lam"), (a_out, "a_out"), (b_out, "b_out")):
+        _dev(t, n, torch.float32)
+    _dev(gates_w, "gates_w")
+    K = taps.shape[1]
+    nb2, bs = gates_w.shape[0], gates_w.shape[1]
+    if yx.shape[1] != 2 * C or taps.shape != (C, K) or x_bias.shape != (C,) or conv_bias.shape != (C,) \
+            or lam.shape != (C,) or nb2 % 2 or (nb2 // 2) * bs != C or gates_w.shape != (nb2, bs, bs) \
+            or gates_b.shape != (nb2, bs) or conv_state.dim() != 3 or conv_state.shape[1:] != (K - 1, C) \
+            or a_out.shape != (nt, C) or b_out.shape != (nt, C):
+        raise KernelError(f"rglru_gates: shapes do not fit {C} channels: yx {tuple(yx.shape)} taps "
+                          f"{tuple(taps.shape)} gates {tuple(gates_w.shape)} state {tuple(conv_state.shape)}")
+    _check(library().ta_rglru_gates(
+        _stream(), c_int(_code(yx.dtype)), c_int(_wcode(gates_w, yx.dtype, "rglru_gates")), _ptr(yx),
+        c_int(stride), c_int(C), _ptr(x_bias), _ptr(taps), _ptr(conv_bias), c_int(K), _ptr(conv_state),
+        _ptr(gates_w), _ptr(gates_b), _ptr(lam), c_float(decay_scale), _ptr(cu_q), _ptr(slots),
+        c_int(batch), c_int(nt), c_int(C), c_int(nb2 // 2), _ptr(a_out), _ptr(b_out)))
+
+
+def rglru_scan(yx: torch.Tensor, channels: int, y_bias, x_bias, a_in, b_in, state, conv_state, cu_q,
+               slots, out: torch.Tensor) -> torch.Tensor:
+    """S_t = a_t S_{t-1} + b_t along every sequence; out_t = S_t * gelu_tanh(y_t + y_bias).
+    ``state`` [slots, C] and ``conv_state`` [slots, K-1, C] (float32) are read and left as the
+    step's last token leaves them."""
+    _dev(yx, "yx", contiguous=False); _dev(out, "out", yx.dtype)
+    nt, stride = _rows2d(yx, "yx")
+    C = channels
+    batch = _step_tables(cu_q, slots, nt, "rglru_scan")
+    for t, n in ((y_bias, "y_bias"), (x_bias, "x_bias"), (a_in, "a_in"), (b_in, "b_in"), (state, "state"),
+                 (conv_state, "conv_state")):
+        _dev(t, n, torch.float32)
+    if yx.shape[1] != 2 * C or out.shape != (nt, C) or a_in.shape != (nt, C) or b_in.shape != (nt, C) \
+            or state.dim() != 2 or state.shape[1] != C or conv_state.dim() != 3 or conv_state.shape[2] != C \
+            or conv_state.shape[0] != state.shape[0]:
+        raise KernelError(f"rglru_scan: shapes do not fit {C} channels")
+    _check(library().ta_rglru_scan(
+        _stream(), c_int(_code(yx.dtype)), _ptr(yx), c_int(stride), c_int(C), _ptr(y_bias), _ptr(x_bias),
+        _ptr(a_in), _ptr(b_in), _ptr(state), _ptr(conv_state), c_int(conv_state.shape[1] + 1), _ptr(cu_q),
+        _ptr(slots), c_int(batch), c_int(C), _ptr(out)))
+    return out
+
+
+def gla_recurrent(proj: torch.Tensor, heads: int, key_dim: int, value_dim: int, rank: int, a2, a2_bias,
+                  tau: float, state: torch.Tensor, cu_q, slots, o_out: torch.Tensor) -> torch.Tensor:
+    """Gated linear attention along every sequence. proj [nt, 2*H*dk + 2*H*dv + rank]: q, k, v,
+    the output gate and the low-rank decay input, in that order. Per head S <- diag(alpha) S +
+    k v^T with alpha = sigmoid(a2 @ low + a2_bias)^(1/tau), o = S^T (q / sqrt(dk)). ``state``
+    [slots, H, dk, dv] float32; o_out [nt, H, dv] float32."""
+    _dev(proj, "proj", contiguous=False)
+    nt, stride = _rows2d(proj, "proj")
+    H, dk, dv = heads, key_dim, value_dim
+    batch = _step_tables(cu_q, slots, nt, "gla_recurrent")
+    _dev(a2, "a2"); _dev(a2_bias, "a2_bias", torch.float32); _dev(state, "state", torch.float32)
+    _dev(o_out, "o_out", torch.float32)
+    if proj.shape[1] != 2 * H * dk + 2 * H * dv + rank or a2.shape != (H * dk, rank) \
+            or a2_bias.shape != (H * dk,) or state.dim() != 4 or state.shape[1:] != (H, dk, dv) \
+            or o_out.shape != (nt, H, dv):
+        raise KernelError(f"gla_recurrent: shapes do not fit {H} heads of {dk} / {dv}, rank {rank}: "
+                          f"proj {tuple(proj.shape)} a2 {tuple(a2.shape)} state {tuple(state.shape)}")
+    _check(library().ta_gla_recurrent(
+        _stream(), c_int(_code(proj.dtype)), c_int(_wcode(a2, proj.dtype, "gla_recurrent")), _ptr(proj),
+        c_int(stride), c_int(0), c_int(H * dk), c_int(2 * H * dk), c_int(2 * H * dk + 2 * H * dv),
+        c_int(rank), _ptr(a2), _ptr(a2_bias), c_float(1.0 / tau), c_float(float(dk) ** -0.5), _ptr(state),
+        _ptr(cu_q), _ptr(slots), c_int(batch), c_int(H), c_int(dk), c_int(dv), _ptr(o_out)))
+    return o_out
+
+
+def gla_out(o: torch.Tensor, proj: torch.Tensor, heads: int, key_dim: int, value_dim: int, weight,
+            eps: float, out: torch.Tensor) -> torch.Tensor:
+    """out = rms_norm(o per head over dv) * weight * silu(gate), the gate being the fourth part
+    of the rows of ``proj`` (see ``gla_recurrent``)."""
+    _dev(o, "o", torch.float32); _dev(proj, "proj", contiguous=False); _dev(out, "out", proj.dtype)
+    _dev(weight, "weight", torch.float32)
+    nt, stride = _rows2d(proj, "proj")
+    H, dk, dv = heads, key_dim, value_dim
+    if o.shape != (nt, H, dv) or out.shape != (nt, H * dv) or weight.shape != (dv,) \
+            or proj.shape[1] < 2 * H * dk + 2 * H * dv:
+        raise KernelError(f"gla_out: o {tuple(o.shape)} out {tuple(out.shape)} weight {tuple(weight.shape)}")
+    _check(library().ta_gla_out(_stream(), c_int(_code(proj.dtype)), _ptr(o), _ptr(proj), c_int(stride),
+                                c_int(2 * H * dk + H * dv), _ptr(weight), c_float(eps), c_int(nt), c_int(H),
+                                c_int(dv), _ptr(out)))
+    return out

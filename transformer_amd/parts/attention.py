@@ -129,3 +129,79 @@ class CachedAttention(Part):
 
 
 register_part("attention", CachedAttention)
+
+
+class NormedAttention(Part):
+    """Attention whose q and k are RMS-normed over the whole projection, rotated on part of
+    every head, and whose values have a width of their own and may be mixed with the values
+    an earlier layer formed for the same token (``NormedAttentionSpec``).
+
+    One merged product gives [q | k | v]; ``kernels.qk_prepare`` does norm, rotation, value
+    mixing and the cache write in one pass; attention over the paged cache follows, then the
+    output projection. The values a "source" layer formed stay in ``ctx.shared`` for the
+    step's later layers."""
+    graph_safe = True
+    _SHARED = "attention_normed.source_values"
+
+    def __init__(self, spec, dtype, device):
+        s = spec
+        if s.num_heads % s.num_kv_heads:
+            raise PartError(f"{s.num_heads} heads do not divide into {s.num_kv_heads} kv heads")
+        if not (1 <= s.key_dim <= 256 and 1 <= s.value_dim <= 256):
+            raise PartError(f"attention takes key and value widths in [1, 256], not {s.key_dim} / {s.value_dim}")
+        if s.rot_dims % 2 or not 0 <= s.rot_dims <= s.key_dim:
+            raise PartError(f"{s.rot_dims} rotated coordinates do not fit heads of {s.key_dim}")
+        if s.value_mix not in (None, "source", "mix"):
+            raise PartError(f"unknown value_mix {s.value_mix!r}")
+        if s.window is not None and s.window < 1:
+            raise PartError(f"attention window must be >= 1, got {s.window}")
+        self.spec, self.dtype = s, dtype
+        self.nq, self.nkv, self.dk, self.dv = s.num_heads, s.num_kv_heads, s.key_dim, s.value_dim
+        self.width = (self.nq + self.nkv) * self.dk + self.nkv * self.dv
+        self.rotary = None
+        if s.rot_dims:
+            from ..config.spec import PositionSpec
+            self.rotary = build_part(PositionSpec(head_dim=s.rot_dims, theta=s.rot_base, style="half"),
+                                     dtype, device)
+
+    def params(self):
+        s = self.spec
+        p = {"qkv.weight": Param((self.width, s.hidden), "matrix"),
+             "out.weight": Param((s.hidden, self.nq * self.dv), "matrix")}
+        if s.qk_norm:
+            p["q_norm.weight"] = Param((self.nq * self.dk,), "vector", init="around_one")
+            p["k_norm.weight"] = Param((self.nkv * self.dk,), "vector", init="around_one")
+        if s.value_mix is not None:
+            p["value_mix"] = Param((), "vector", init="zero")    # a source holds it too, unused
+        return p
+
+    def cache_need(self):
+        return KVNeed(self.nkv, self.dk, self.spec.window, self.dv)
+
+    def run(self, h, ctx, cache, layer, writes_cache=True):
+        s, nt = self.spec, h.shape[0]
+        qkv = linear(h, self.w["qkv.weight"], ctx.ws.take("attention.qkv", (nt, self.width), self.dtype))
+        kc, vc, group = cache.layer_kv(layer)
+        meta = ctx.kv[group]
+        nv = self.nkv * self.dv
+        keep = first = mix = None
+        if s.value_mix == "source":
+            keep = ctx.ws.take(self._SHARED, (nt, nv), self.dtype)
+            ctx.shared[self._SHARED] = keep
+        elif s.value_mix == "mix":
+            first = ctx.shared.get(self._SHARED)
+            if first is None or first.shape != (nt, nv):
+                raise PartError("a layer that mixes values runs after the layer that is their source, "
+                                "with values of the same width")
+            mix = self.w["value_mix"].reshape(1)
+        angles = self.rotary.angles(ctx) if self.rotary is not None else None
+        kernels.qk_prepare(qkv, self.nq, self.nkv, self.dk, self.dv, float(s.eps),
+                           self.w.get("q_norm.weight"), self.w.get("k_norm.weight"), angles, s.rot_dims,
+                           mix, first, keep, meta.dest if writes_cache else None, kc, vc)
+        o = ctx.ws.take("attention.o", (nt, self.nq * self.dv), self.dtype)
+        kernels.attention_generic_dv(qkv, o, kc, vc, meta.block_table, ctx.cu_q, ctx.pos0, ctx.max_qlen,
+                                     self.nq, self.nkv, self.dk, self.dv, float(s.scale), s.window)
+        return linear_delta(o, self.w["out.weight"], ctx.ws, "attention.delta"), None
+
+
+register_part("attention_normed", NormedAttention)

@@ -102,3 +102,97 @@ class PreNormBlock(Part):
 
 
 register_part("prenorm", PreNormBlock)
+
+
+class GatedPreNormBlock(Part):
+    """x += mult * gate1 * mixer(shift(norm1(x))); x += mult * gate2 * ffn(norm2(x)).
+
+    The gate of a sublayer is sigmoid(W h + b) of the sublayer's normed input h; the mixer reads
+    the token-shifted rows. What a sublayer adds travels as a ``kernels.GatedDelta`` to the
+    next norm (of this block or of the next, or the model's last), which does the add in
+    float32 and normalises in the same pass. The shift keeps the sequence's last normed row
+    between steps (a state row of its own, before the mixer's needs)."""
+    folds_norms = False
+
+    def __init__(self, spec, dtype, device):
+        self.spec, self.dtype = spec, dtype
+        self.hidden = spec.hidden
+        self.norm1 = build_part(spec.norm1, dtype, device)
+        self.mixer = build_part(spec.mixer, dtype, device)
+        self.norm2 = build_part(spec.norm2, dtype, device) if spec.ffn is not None else None
+        self.ffn = build_part(spec.ffn, dtype, device) if spec.ffn is not None else None
+
+    def children(self):
+        c = {"norm1": self.norm1, "mixer": self.mixer}
+        if self.ffn is not None:
+            c.update(norm2=self.norm2, ffn=self.ffn)
+        return c
+
+    def params(self):
+        from ..weights.loader import Param
+        d, p = self.hidden, {}
+        if self.spec.token_shift:
+            p["shift"] = Param((d,), "vector", init="zero")
+        if self.spec.gated:
+            p["gate1.weight"], p["gate1.bias"] = Param((d, d), "matrix"), Param((d,), "vector")
+            if self.ffn is not None:
+                p["gate2.weight"], p["gate2.bias"] = Param((d, d), "matrix"), Param((d,), "vector")
+        return p
+
+    def _mixer_needs(self):
+        need = self.mixer.cache_need()
+        if need is None:
+            return []
+        return list(need) if isinstance(need, (list, tuple)) else [need]
+
+    def cache_need(self):
+        from ..cache.storage import StateNeed
+        own = [StateNeed((self.hidden,), torch.float32)] if self.spec.token_shift else []
+        return own + self._mixer_needs()
+
+    def step_planner(self):
+        f = getattr(self.mixer, "step_planner", None)
+        return f() if f is not None else None
+
+    @property
+    def graph_safe(self) -> bool:
+        return all(getattr(p, "graph_safe", False) for p in self.children().values())
+
+    def _gate(self, h, which, ctx):
+        if not self.spec.gated:
+            return None, None
+        from .linear import linear
+        g = linear(h, self.w[which + ".weight"],
+                   ctx.ws.take("block." + which, (h.shape[0], self.hidden), torch.float32))
+        return g, self.w[which + ".bias"]
+
+    def run(self, x, pending, ctx, cache, layer, writes_cache=True, after=None):
+        s = self.spec
+        h = ctx.ws.take("block.h", x.shape, self.dtype)
+        with span(ctx, "norm"):
+            self.norm1.run(x, h, pending[0], pending[1])
+        layers = list(layer) if isinstance(layer, (list, tuple)) else ([] if layer is None else [layer])
+        with span(ctx, "gate"):
+            gate, gbias = self._gate(h, "gate1", ctx)
+            hs = h
+            if s.token_shift:
+                hs = kernels.token_shift(h, ctx.ws.take("block.hs", x.shape, self.dtype), self.w["shift"],
+                                         cache.layer_state(layers.pop(0)), ctx.cu_q, ctx.slots)
+        need = self.mixer.cache_need()
+        mixer_layer = None if need is None else tuple(layers) if isinstance(need, (list, tuple)) \
+            else layers[0]
+        with span(ctx, "mixer"):
+            delta, bias = self.mixer.run(hs, ctx, cache, mixer_layer, writes_cache)
+        pending = (kernels.GatedDelta(delta, bias, gate, gbias, s.mult), None)
+        if self.ffn is None:
+            return pending
+        with span(ctx, "norm"):
+            self.norm2.run(x, h, pending[0], pending[1])
+        with span(ctx, "gate"):
+            gate, gbias = self._gate(h, "gate2", ctx)
+        with span(ctx, "ffn"):
+            delta, bias = self.ffn.run(h, ctx)
+        return (kernels.GatedDelta(delta, bias, gate, gbias, s.mult), None)
+
+
+register_part("gated_prenorm", GatedPreNormBlock)

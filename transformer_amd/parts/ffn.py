@@ -11,7 +11,7 @@ import torch
 
 from .. import kernels
 from ..weights.loader import Param
-from .base import Part, register_part
+from .base import Part, PartError, register_part
 from .linear import adds_in_place, linear, linear_delta
 
 
@@ -65,4 +65,34 @@ class SwiGLU(Part):
                 self.w.get("down.bias"))
 
 
+class GLU(SwiGLU):
+    """The same feed-forward with the activation as a parameter of the spec ("silu",
+    "gelu_tanh"). Silu takes every path of ``SwiGLU`` (the products that apply it themselves
+    included); another activation runs the product and then the activation's kernel."""
+
+    def __init__(self, spec, dtype, device):
+        super().__init__(spec, dtype, device)
+        if spec.activation not in ("silu", "gelu_tanh"):
+            raise PartError(f"unknown feed-forward activation {spec.activation!r}")
+        self.activation = spec.activation
+
+    def takes_scaled(self, nt: int) -> bool:
+        return self.activation == "silu" and super().takes_scaled(nt)
+
+    def run(self, h, ctx, scale=None, fold=None, into=None):
+        if self.activation == "silu":
+            return super().run(h, ctx, scale=scale, fold=fold, into=into)
+        s, nt = self.spec, h.shape[0]
+        gu = linear(h, self.w["gate_up.weight"],
+                    ctx.ws.take("swiglu.gate_up", (nt, 2 * s.intermediate), self.dtype))
+        act = kernels.glu(gu, ctx.ws.take("swiglu.act", (nt, s.intermediate), self.dtype),
+                          self.activation, self.w.get("gate_up.bias"))
+        if fold is not None:
+            kernels.gemm_skinny(act, self.w["down.weight"], None, bias=self.w.get("down.bias"), fold=fold)
+            return None
+        return (linear_delta(act, self.w["down.weight"], ctx.ws, "swiglu.delta", into=into),
+                self.w.get("down.bias"))
+
+
 register_part("swiglu", SwiGLU)
+register_part("glu", GLU)

@@ -29,14 +29,37 @@ class RMSNorm(Part):
     def run(self, x: torch.Tensor, out: torch.Tensor, delta: Optional[torch.Tensor] = None,
             delta_bias: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None):
         """x: float32 [nt, size], updated in place by the pending delta unless
-        ``rows`` selects the rows to normalise. out: engine dtype."""
-        return kernels.add_rmsnorm(x, self.w["weight"], self.eps, out, delta, delta_bias, rows)
+        ``rows`` selects the rows to normalise. out: engine dtype. ``delta`` may be a
+        ``kernels.GatedDelta`` (what a gated sublayer leaves to be added)."""
+        if isinstance(delta, kernels.GatedDelta):
+            return kernels.gated_add_rmsnorm(x, self.gain(), self.eps, out, delta, rows)
+        return kernels.add_rmsnorm(x, self.gain(), self.eps, out, delta, delta_bias, rows)
+
+    def gain(self) -> torch.Tensor:
+        """The weight per coordinate, float32 [size]."""
+        return self.w["weight"]
 
     def fold(self, x: torch.Tensor, out: torch.Tensor, ctx) -> "kernels.NormFold":
         """For the few-rows product in front of this norm, which then does the add and the
         sums of squares itself; ``.scale()`` of the result goes to the product behind it."""
         parts = ctx.ws.take("norm.parts", kernels.NormFold.parts_shape(self.size), torch.float32)
-        return kernels.NormFold(x, self.w["weight"], self.eps, out, parts)
+        return kernels.NormFold(x, self.gain(), self.eps, out, parts)
+
+
+class ScalarRMSNorm(RMSNorm):
+    """The same norm with one gain for all coordinates: the parameter is a 0-d tensor, and the
+    kernels get it spread over a row once, when the weights are bound."""
+
+    def params(self):
+        return {"weight": Param((), "vector", init="around_one")}
+
+    def bind(self, tensors):
+        super().bind(tensors)
+        self._gain = tensors["weight"].to(torch.float32).reshape(1).expand(self.size).contiguous()
+
+    def gain(self):
+        return self._gain
 
 
 register_part("rmsnorm", RMSNorm)
+register_part("rmsnorm_scalar", ScalarRMSNorm)

@@ -1,0 +1,102 @@
+"""Mixers that keep a state of fixed size per sequence instead of a cache of keys.
+
+``DiagonalRecurrence``: a gated linear recurrence per channel behind a short causal
+convolution (the recurrent block of De et al., "Griffin: Mixing Gated Linear Recurrences with
+Local Attention for Efficient Language Models"). ``GatedLinearAttention``: a matrix state per
+head with a decay per key channel. Both walk a sequence's tokens in order in float32, so the
+result does not depend on how the sequence was cut into steps; a step's products (the input
+and output projections) are the framework's usual ones.
+"""
+from __future__ import annotations
+
+import torch
+
+from .. import kernels
+from ..cache.storage import StateNeed
+from ..weights.loader import Param
+from .base import Part, PartError, register_part
+from .linear import linear, linear_delta
+
+
+class DiagonalRecurrence(Part):
+    graph_safe = True
+
+    def __init__(self, spec, dtype, device):
+        s = spec
+        if s.channels < 1 or s.blocks < 1 or s.channels % s.blocks:
+            raise PartError(f"{s.channels} channels do not divide into {s.blocks} blocks")
+        if s.taps < 1:
+            raise PartError(f"a convolution needs at least one tap, got {s.taps}")
+        self.spec, self.dtype = s, dtype
+
+    def params(self):
+        s = self.spec
+        C, bs = s.channels, s.channels // s.blocks
+        return {"in.weight": Param((2 * C, s.hidden), "matrix"),       # y branch, then x branch
+                "in.bias": Param((2 * C,), "vector"),
+                "conv.weight": Param((C, s.taps), "vector"),
+                "conv.bias": Param((C,), "vector"),
+                "gates.weight": Param((2 * s.blocks, bs, bs), "matrix"),   # recurrence gate, then input gate
+                "gates.bias": Param((2 * s.blocks, bs), "vector"),
+                "lam": Param((C,), "vector"),
+                "out.weight": Param((s.hidden, C), "matrix")}
+
+    def cache_need(self):
+        s = self.spec
+        return [StateNeed((s.channels,), torch.float32), StateNeed((s.taps - 1, s.channels), torch.float32)]
+
+    def run(self, h, ctx, cache, layer, writes_cache=True):
+        s, nt, C = self.spec, h.shape[0], self.spec.channels
+        state, conv_state = cache.layer_state(layer[0]), cache.layer_state(layer[1])
+        yx = linear(h, self.w["in.weight"], ctx.ws.take("recurrence.in", (nt, 2 * C), self.dtype))
+        a = ctx.ws.take("recurrence.a", (nt, C), torch.float32)
+        b = ctx.ws.take("recurrence.b", (nt, C), torch.float32)
+        bias = self.w["in.bias"]
+        kernels.rglru_gates(yx, C, bias[C:], self.w["conv.weight"], self.w["conv.bias"], conv_state,
+                            self.w["gates.weight"], self.w["gates.bias"], self.w["lam"],
+                            float(s.decay_scale), ctx.cu_q, ctx.slots, a, b)
+        o = kernels.rglru_scan(yx, C, bias[:C], bias[C:], a, b, state, conv_state, ctx.cu_q, ctx.slots,
+                               ctx.ws.take("recurrence.o", (nt, C), self.dtype))
+        return linear_delta(o, self.w["out.weight"], ctx.ws, "recurrence.delta"), None
+
+
+class GatedLinearAttention(Part):
+    graph_safe = True
+
+    def __init__(self, spec, dtype, device):
+        s = spec
+        if not (1 <= s.key_dim <= 256 and s.value_dim >= 1 and s.rank >= 1 and s.num_heads >= 1):
+            raise PartError(f"gated linear attention: heads {s.num_heads} of {s.key_dim} / {s.value_dim}, "
+                            f"rank {s.rank}")
+        if not s.tau > 0:
+            raise PartError(f"gated linear attention: tau must be positive, got {s.tau}")
+        self.spec, self.dtype = s, dtype
+        self.width = 2 * s.num_heads * s.key_dim + 2 * s.num_heads * s.value_dim + s.rank
+
+    def params(self):
+        s = self.spec
+        H, dk, dv = s.num_heads, s.key_dim, s.value_dim
+        return {"in.weight": Param((self.width, s.hidden), "matrix"),     # q, k, v, gate, decay input
+                "decay.weight": Param((H * dk, s.rank), "matrix"),
+                "decay.bias": Param((H * dk,), "vector"),
+                "norm.weight": Param((dv,), "vector", init="around_one"),
+                "out.weight": Param((s.hidden, H * dv), "matrix")}
+
+    def cache_need(self):
+        s = self.spec
+        return StateNeed((s.num_heads, s.key_dim, s.value_dim), torch.float32)
+
+    def run(self, h, ctx, cache, layer, writes_cache=True):
+        s, nt = self.spec, h.shape[0]
+        H, dk, dv = s.num_heads, s.key_dim, s.value_dim
+        proj = linear(h, self.w["in.weight"], ctx.ws.take("gla.in", (nt, self.width), self.dtype))
+        o = kernels.gla_recurrent(proj, H, dk, dv, s.rank, self.w["decay.weight"], self.w["decay.bias"],
+                                  float(s.tau), cache.layer_state(layer), ctx.cu_q, ctx.slots,
+                                  ctx.ws.take("gla.o", (nt, H, dv), torch.float32))
+        g = kernels.gla_out(o, proj, H, dk, dv, self.w["norm.weight"], float(s.eps),
+                            ctx.ws.take("gla.gated", (nt, H * dv), self.dtype))
+        return linear_delta(g, self.w["out.weight"], ctx.ws, "gla.delta"), None
+
+
+register_part("diagonal_recurrence", DiagonalRecurrence)
+register_part("gated_linear_attention", GatedLinearAttention)
