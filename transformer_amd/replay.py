@@ -33,7 +33,10 @@ class TraceError(ValueError):
 class Replayer:
     def __init__(self, model, max_tokens: int, out_dir):
         self.model = model
-        self.cache = model.new_cache(max_tokens)
+        # the cache hands out whole pages: every live request may hold a page that is not full,
+        # so there is room for that beside the tokens themselves (up to 64 requests at once)
+        from .kernels import PAGE
+        self.cache = model.new_cache(max_tokens + PAGE * min(max(max_tokens, 1), 64))
         self.out = Path(out_dir)
         self.out.mkdir(parents=True, exist_ok=True)
         (self.out / "index.jsonl").write_text("")
@@ -83,7 +86,7 @@ def main(argv=None) -> int:
     ap.add_argument("--dtype", required=True, choices=["bfloat16", "float32"])
     ap.add_argument("--out", required=True, help="folder for <step>.f32 files")
     ap.add_argument("--max-tokens", type=int, required=True,
-                    help="most tokens live requests hold at any time (each rounded up to 64)")
+                    help="most tokens live requests hold at any time")
     ap.add_argument("--device", default="cuda:0")
     args = ap.parse_args(argv)
     from .api import load_model
