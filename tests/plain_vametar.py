@@ -15,7 +15,32 @@ from pathlib import Path
 
 import numpy as np
 
-from plain_llama import read_safetensors, write_safetensors  # noqa: F401  (the suite's own file code)
+from plain_llama import read_safetensors, round_bf16  # noqa: F401  (the suite's own file code)
+
+
+def write_safetensors(path, tensors: dict, dtype="BF16"):
+    """name -> float ndarray (0-d included), stored as F32 or BF16."""
+    import struct
+    header, blobs, off = {}, [], 0
+    for name, a in tensors.items():
+        a = np.asarray(a, dtype=np.float64)
+        flat = a.reshape(-1)
+        if dtype == "F32":
+            b = flat.astype("<f4").tobytes()
+        elif dtype == "BF16":
+            b = (round_bf16(flat).astype(np.float32).view(np.uint32) >> 16).astype("<u2").tobytes()
+        else:
+            raise ValueError(dtype)
+        header[name] = {"dtype": dtype, "shape": list(a.shape), "data_offsets": [off, off + len(b)]}
+        blobs.append(b)
+        off += len(b)
+    h = json.dumps(header, separators=(",", ":")).encode()
+    h += b" " * ((8 - len(h) % 8) % 8)
+    with open(path, "wb") as f:
+        f.write(struct.pack("<Q", len(h)))
+        f.write(h)
+        for b in blobs:
+            f.write(b)
 
 
 # --------------------------------------------------------------------------
@@ -289,7 +314,6 @@ def tensor_shapes(c):
 def random_weights(c, seed, edit=None):
     """float64 weights, already rounded to bfloat16 values so that a bfloat16 file holds them
     exactly. Matrices ~ N(0, 1/sqrt(in)); gains near 1; shifts and mixing weights in (0, 1)."""
-    from plain_llama import round_bf16
     rng = np.random.default_rng(seed)
     w = {}
     for name, shape in tensor_shapes(c).items():

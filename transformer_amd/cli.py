@@ -229,14 +229,15 @@ def main(argv: Optional[Sequence[str]] = None) -> int:
         from .weights.random_init import write_random_model
         from .config.shapes import SHAPES
         d = dict(SHAPES[a.config][1]) if a.config in SHAPES else json.loads(Path(a.config).read_text())
-        if a.layers is not None:
-            d["num_hidden_layers"] = a.layers
         arch = architecture_of_config_json(d)
+        cfg = arch.config_from_dict(d)
+        if a.layers is not None:
+            cfg = cfg.with_layers(a.layers)
         if a.on_gpu:
             import time
             from .api import random_model, save_model
             from .engine.generate import generate
-            model = random_model(arch.config_from_dict(d), a.seed, a.storage, architecture=arch.name)
+            model = random_model(cfg, a.seed, a.storage, architecture=arch.name)
             t0 = time.time()
             save_model(model, a.out, metadata={"seed": a.seed})
             print(f"[transformer_amd] wrote {model.weight_bytes() / 1e9:.2f} GB in {time.time() - t0:.1f} s",
@@ -245,7 +246,7 @@ def main(argv: Optional[Sequence[str]] = None) -> int:
                 toks = prompt_to_tokens(a.probe, a.out)
                 print("probe:", " ".join(map(str, generate(model, [toks], 8, stop_ids=[]).tokens[0])))
         else:
-            write_random_model(a.out, arch.config_from_dict(d), a.seed, a.storage, architecture=arch.name)
+            write_random_model(a.out, cfg, a.seed, a.storage, architecture=arch.name)
         print(a.out)
         return 0
     if a.cmd == "replay":

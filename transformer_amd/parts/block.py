@@ -132,7 +132,7 @@ class GatedPreNormBlock(Part):
         from ..weights.loader import Param
         d, p = self.hidden, {}
         if self.spec.token_shift:
-            p["shift"] = Param((d,), "vector", init="zero")
+            p["shift"] = Param((d,), "vector")
         if self.spec.gated:
             p["gate1.weight"], p["gate1.bias"] = Param((d, d), "matrix"), Param((d,), "vector")
             if self.ffn is not None:
