@@ -147,6 +147,121 @@ def prefill_point(model, cfg, dkey, reps, seed, tokens=None, lengths=None):
             "frac": round(fl / pt / (PEAK_TFLOPS[dkey] * 1e12), 4)}
 
 
+# ---------------------------------------------------------------------------------------------
+# --design vametar: the Vametar decoder beside the Llama decoder at equal layer sizes
+
+def vametar_shapes():
+    """Layer sizes that resemble real models' (random weights). Each gives the Vametar mixers'
+    sizes and the Llama layer of the same width, heads and feed-forward."""
+    def shape(width, heads, kv, ff, rec_width, rec_blocks, gla_heads, gla_dim, gla_vdim, vocab):
+        att = {"type": "attention", "mlp": {"kind": "dense", "ff": ff},
+               "mixer": {"heads": heads, "kv_heads": kv, "dim": 128, "vdim": 64, "scale": 128 ** -0.5,
+                         "rot": {"base": 500000.0, "dims": 128}, "v_mix": True}}
+        rec = {"type": "rglru", "mlp": {"kind": "dense", "ff": ff},
+               "mixer": {"width": rec_width, "blocks": rec_blocks, "conv": 4}}
+        gla = {"type": "gla", "mlp": {"kind": "dense", "ff": ff},
+               "mixer": {"heads": gla_heads, "dim": gla_dim, "vdim": gla_vdim, "tau": 16.0, "rank": 16}}
+        base = {"architecture": "Vametar", "vocab": vocab, "width": width, "norm": {"eps": 1e-5},
+                "residual_mult": 0.7, "logit_scale": 2.0,
+                "embedding": {"bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 7}}}
+        llama = {"architectures": ["LlamaForCausalLM"], "model_type": "llama", "hidden_size": width,
+                 "num_attention_heads": heads, "num_key_value_heads": kv, "head_dim": 128,
+                 "intermediate_size": ff, "vocab_size": vocab, "rope_theta": 500000.0, "rms_norm_eps": 1e-5,
+                 "tie_word_embeddings": False, "max_position_embeddings": 1 << 20, "rope_scaling": None}
+        return base, {"attention": att, "rglru": rec, "gla": gla}, llama
+    return {"w2048": shape(2048, 16, 4, 8192, 2560, 10, 16, 64, 128, 32000),
+            "w4096": shape(4096, 32, 8, 14336, 4096, 16, 32, 128, 128, 32000)}
+
+
+def generic_step_bytes(model, contexts):
+    """What a single-token step reads and writes: every matrix once (of the embedding tables
+    only rows), each sequence's keys and values, and its fixed-size state twice."""
+    import torch
+    from transformer_amd.cache.storage import KVNeed, StateNeed
+    w = model.weight_bytes()
+    skip = {model.w["embed"].data_ptr()}
+    if model.w["embed"].data_ptr() != model.w["head"].data_ptr():
+        w -= model.w["embed"].numel() * model.w["embed"].element_size()
+    table = getattr(getattr(model, "after_embed", None), "w", {}).get("table")
+    if table is not None and table.data_ptr() not in skip:
+        w -= table.numel() * table.element_size()
+    item = torch.empty((), dtype=model.dtype).element_size()
+    per_token = per_seq = 0
+    for need in model.cache_needs:
+        if isinstance(need, KVNeed):
+            per_token += need.num_kv_heads * (need.head_dim + need.value_dim) * item
+        elif isinstance(need, StateNeed):
+            n = 1
+            for d in need.shape:
+                n *= d
+            per_seq += 2 * n * torch.empty((), dtype=need.dtype).element_size()
+    return w + sum(contexts) * per_token + len(contexts) * per_seq
+
+
+def generic_prefill_flops(model, T):
+    """2 * T * (entries of every matrix but the embedding tables) plus, for each attention
+    layer, the causal score and value products."""
+    from transformer_amd.cache.storage import KVNeed
+    params = model.all_params()
+    mats = sum(t.numel() for n, t in model.tensors.items()
+               if params[n].role == "matrix" and n not in ("embed.weight", "head.weight", "after_embed.table"))
+    fl = 2 * T * mats + 2 * model.spec.hidden * model.spec.vocab
+    for blk in model.blocks:
+        m = blk.mixer
+        need = m.cache_need()
+        if isinstance(need, KVNeed):
+            heads = getattr(m, "nq")
+            fl += 2 * heads * (need.head_dim + need.value_dim) * (T * (T + 1) // 2)
+    return fl
+
+
+class _Vocab:
+    def __init__(self, vocab):
+        self.vocab = vocab
+
+
+def bench_design(a):
+    """Prefill and decode throughput of Vametar models whose layers are all of one kind, and
+    of the mixed order, beside the Llama decoder with layers of the same width, heads and
+    feed-forward. One JSON line of its own; the default workload is untouched."""
+    import torch
+    import transformer_amd as ta
+    dkey = "bf16" if a.dtype == "bfloat16" else "fp32"
+    layers = a.layers or 8
+    out = {"design": "vametar", "dtype": dkey, "layers": layers, "batch": a.batch,
+           "prefill_tokens": a.prefill_tokens, "data": "synthetic", "sizes": {}}
+    for size, (base, kinds, llama) in vametar_shapes().items():
+        if a.design_size and size not in a.design_size.split(","):
+            continue
+        rows = {}
+        order = ["gla", "attention", "rglru", "attention", "gla"]
+        cases = [("llama", None)] + [(k, [kinds[k]] * layers) for k in ("attention", "rglru", "gla")] + \
+                [("mixed", [kinds[order[i % len(order)]] for i in range(layers)])]
+        for name, lay in cases:
+            if name == "llama":
+                model = ta.random_model(ta.LlamaConfig.from_dict({**llama, "num_hidden_layers": layers}),
+                                        seed=0, dtype=a.dtype)
+            else:
+                model = ta.random_model({**base, "layers": lay}, seed=0, dtype=a.dtype, architecture="Vametar")
+            cfg = _Vocab(model.spec.vocab)
+            dt, ctx, _ = time_decode(model, cfg, a.batch, a.steps, a.warmup, 1, 512, 1024)
+            nbytes = generic_step_bytes(model, ctx)
+            pt = time_prefill(model, cfg, 3, 2, tokens=a.prefill_tokens)
+            fl = generic_prefill_flops(model, a.prefill_tokens)
+            rows[name] = {"decode_tok_s": round(a.batch * a.steps / dt, 1),
+                          "decode_ms_per_step": round(dt / a.steps * 1e3, 4),
+                          "decode_gbs": round(nbytes / (dt / a.steps) / 1e9, 1),
+                          "decode_frac_hbm": round(nbytes / (dt / a.steps) / 1e9 / HBM_GBS, 4),
+                          "prefill_tok_s": round(a.prefill_tokens / pt, 1), "prefill_ms": round(pt * 1e3, 3),
+                          "prefill_frac_matrix_peak": round(fl / pt / (PEAK_TFLOPS[dkey] * 1e12), 4)}
+            del model
+            torch.cuda.empty_cache()
+            print(f"[bench] {size} {name}: {rows[name]}", file=sys.stderr, flush=True)
+        out["sizes"][size] = rows
+    print(json.dumps(out))
+    return 0
+
+
 def read_probe_gbs(device, nbytes=1 << 30, workgroups=2048, reps=5):
     """GB/s of a kernel that only reads: the machine's own ceiling for the weight streams of a
     decode step (the roofline of the line is the published 8 TB/s; this says how much of the
@@ -188,7 +303,13 @@ def main():
                     help="tokens of the prompt whose step is timed (the line's \"prefill\")")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the 2,048-token prefill (for profiling); prints its own line")
+    ap.add_argument("--design", default=None, choices=["vametar"],
+                    help="instead of the default workload: prefill and decode of this design at a few "
+                         "layer sizes, beside the Llama decoder at the same sizes (a line of its own)")
+    ap.add_argument("--design-size", default=None, help="with --design: only these sizes (w2048,w4096)")
     a = ap.parse_args()
+    if a.design and a.gpus == 1:
+        return bench_design(a)
     if a.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {a.gpus} is not supported by this engine")
         return 2

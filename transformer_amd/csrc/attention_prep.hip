@@ -6,7 +6,7 @@
 //   the first `rot` coordinates of every head of q and k are rotated in pairs (i, i + rot/2)
 //   v <- (1 - lambda) v + lambda v_first      (where the layer mixes in the values of an earlier one)
 //   q is written back in place; k and v go to the paged cache (keys [pages][kv heads][PAGE][dk],
-//   values [pages][kv heads][dv][PAGE]).
+//   values [pages][kv heads][dvs][PAGE], dvs >= dv, rows dv.. of a token zero).
 //
 // One workgroup per token. Everything is float32 until the single rounding of each result.
 #include "common.h"
@@ -17,7 +17,7 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
     float eps, int normed, const float* __restrict__ angles, int rot,
     const float* __restrict__ lambda, const T* __restrict__ v_first, T* __restrict__ v_keep,
     const int* __restrict__ dest, T* __restrict__ kcache, T* __restrict__ vcache,
-    int nh, int nkv, int dk, int dv) {
+    int nh, int nkv, int dk, int dv, int dvs) {
   extern __shared__ float buf[];          // [nh*dk + nkv*dk]
   __shared__ float red[8];
   const int t = blockIdx.x;
@@ -73,7 +73,15 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
     if (v_first) v = (1.0f - lam) * v + lam * to_f32(v_first[(size_t)t * nv + i]);
     if (dest) {
       const int g = i / dv, c = i - g * dv;
-      vcache[(((size_t)page * nkv + g) * dv + c) * TA_PAGE + off] = from_f32<T>(v);
+      vcache[(((size_t)page * nkv + g) * dvs + c) * TA_PAGE + off] = from_f32<T>(v);
+    }
+  }
+  // a cache whose value rows are wider than the values (dvs > dv) holds zeros there
+  if (dest && dvs > dv) {
+    const int pad = dvs - dv;
+    for (int i = threadIdx.x; i < nkv * pad; i += 256) {
+      const int g = i / pad, c = dv + (i - g * pad);
+      vcache[(((size_t)page * nkv + g) * dvs + c) * TA_PAGE + off] = from_f32<T>(0.f);
     }
   }
 }
@@ -85,13 +93,15 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
 extern "C" int ta_qk_prepare(hipStream_t stream, int dtype, void* qkv, int stride, const float* wq,
                              const float* wk, float eps, int normed, const float* angles, int rot,
                              const float* lambda, const void* v_first, void* v_keep, const int* dest,
-                             void* kcache, void* vcache, int nt, int nh, int nkv, int dk, int dv) {
+                             void* kcache, void* vcache, int nt, int nh, int nkv, int dk, int dv,
+                             int dvs) {
   TA_REQUIRE(nt >= 0 && nh > 0 && nkv > 0 && dk > 0 && dv > 0, "ta_qk_prepare: bad sizes");
   TA_REQUIRE(stride >= (nh + nkv) * dk + nkv * dv, "ta_qk_prepare: row stride %d too small", stride);
   TA_REQUIRE(rot >= 0 && rot <= dk && rot % 2 == 0, "ta_qk_prepare: %d rotated coordinates of %d", rot, dk);
   TA_REQUIRE((lambda == nullptr) == (v_first == nullptr), "ta_qk_prepare: lambda and v_first go together");
   TA_REQUIRE(!normed || (wq && wk), "ta_qk_prepare: norm weights missing");
   TA_REQUIRE(!dest || (kcache && vcache), "ta_qk_prepare: cache layer missing");
+  TA_REQUIRE(dvs >= dv, "ta_qk_prepare: cache rows of %d cannot hold values of %d", dvs, dv);
   const size_t lds = (size_t)(nh + nkv) * dk * sizeof(float);
   TA_REQUIRE(lds <= 60000, "ta_qk_prepare: %d + %d heads of %d do not fit", nh, nkv, dk);
   if (nt == 0) return 0;
@@ -99,11 +109,11 @@ extern "C" int ta_qk_prepare(hipStream_t stream, int dtype, void* qkv, int strid
   if (dtype == TA_F32)
     qk_prepare_kernel<float><<<nt, 256, lds, stream>>>(
         (float*)qkv, stride, wq, wk, eps, normed, angles, rot, lambda, (const float*)v_first, (float*)v_keep,
-        dest, (float*)kcache, (float*)vcache, nh, nkv, dk, dv);
+        dest, (float*)kcache, (float*)vcache, nh, nkv, dk, dv, dvs);
   else if (dtype == TA_BF16)
     qk_prepare_kernel<bf16_t><<<nt, 256, lds, stream>>>(
         (bf16_t*)qkv, stride, wq, wk, eps, normed, angles, rot, lambda, (const bf16_t*)v_first, (bf16_t*)v_keep,
-        dest, (bf16_t*)kcache, (bf16_t*)vcache, nh, nkv, dk, dv);
+        dest, (bf16_t*)kcache, (bf16_t*)vcache, nh, nkv, dk, dv, dvs);
   else
     return ta_fail("ta_qk_prepare: unknown dtype %d", dtype);
   return ta_check_launch("ta_qk_prepare");

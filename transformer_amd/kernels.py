@@ -959,7 +959,8 @@ def qk_prepare(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, key_dim: in
     over all their heads at once (weights given: else none), rotation of the first ``rot``
     coordinates of every head by ``angles`` [nt, rot/2, 2], v <- (1 - mix) v + mix v_first,
     q written back in place, k and v stored at ``dest`` into the cache layer. ``v_keep``
-    receives the values before mixing."""
+    receives the values before mixing. The cache's value rows may be wider than the values
+    (vcache [pages, nkv, dvs, PAGE], dvs >= value_dim): the rest of a token's column is zeroed."""
     _dev(qkv, "qkv", contiguous=False)
     nt, stride = _rows2d(qkv, "qkv")
     nq, nk, nv = num_heads * key_dim, num_kv_heads * key_dim, num_kv_heads * value_dim
@@ -988,14 +989,18 @@ def qk_prepare(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, key_dim: in
             raise KernelError(f"qk_prepare: v_keep is {tuple(v_keep.shape)}, expected {(nt, nv)}")
     if dest is not None:
         _dev(dest, "dest", torch.int32); _dev(kcache, "kcache", qkv.dtype); _dev(vcache, "vcache", qkv.dtype)
-        _check_cache_layer("qk_prepare", kcache, vcache, num_kv_heads, key_dim, value_dim)
+        store_dim = vcache.shape[2] if vcache.dim() == 4 else -1
+        if store_dim < value_dim:
+            raise KernelError(f"qk_prepare: cache value rows of {store_dim} cannot hold values of {value_dim}")
+        _check_cache_layer("qk_prepare", kcache, vcache, num_kv_heads, key_dim, store_dim)
         if dest.numel() != nt:
             raise KernelError("qk_prepare: dest must hold one entry per token")
     _check(library().ta_qk_prepare(
         _stream(), c_int(_code(qkv.dtype)), _ptr(qkv), c_int(stride), _ptr(q_weight), _ptr(k_weight),
         c_float(eps), c_int(int(normed)), _ptr(angles), c_int(rot), _ptr(mix), _ptr(v_first), _ptr(v_keep),
         _ptr(dest), _ptr(kcache if dest is not None else None), _ptr(vcache if dest is not None else None),
-        c_int(nt), c_int(num_heads), c_int(num_kv_heads), c_int(key_dim), c_int(value_dim)))
+        c_int(nt), c_int(num_heads), c_int(num_kv_heads), c_int(key_dim), c_int(value_dim),
+        c_int(store_dim if dest is not None else value_dim)))
     return qkv
 
 

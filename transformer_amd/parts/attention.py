@@ -175,8 +175,31 @@ class NormedAttention(Part):
             p["value_mix"] = Param((), "vector", init="zero")    # a source holds it too, unused
         return p
 
+    # bfloat16 with a key width the matrix-core kernels take and values no wider than the keys:
+    # the cache keeps value rows of the keys' width (the rest zero), so that the kernels for
+    # equal widths serve prompts and single tokens, and the output projection reads the heads'
+    # rows through a copy of its matrix with zero columns in the same places. Everything else
+    # (float32, other widths) runs the vector-ALU kernel on values of their own width.
+    def _on_matrix_cores(self) -> bool:
+        return (self.dtype == torch.bfloat16 and self.dk % 32 == 0 and 32 <= self.dk <= 256
+                and self.dv <= self.dk)
+
     def cache_need(self):
-        return KVNeed(self.nkv, self.dk, self.spec.window, self.dv)
+        return KVNeed(self.nkv, self.dk, self.spec.window, self.dk if self._on_matrix_cores() else self.dv)
+
+    def step_planner(self):
+        if self._on_matrix_cores() and kernels.keys_kernel_fits(self.nq, self.nkv, self.dk):
+            return KeyUnitPlanner(self.nkv)
+        return None
+
+    def bind(self, tensors):
+        super().bind(tensors)
+        self.out_wide = None
+        if self._on_matrix_cores() and self.dv < self.dk and tensors["out.weight"].is_cuda:
+            w = tensors["out.weight"]
+            wide = torch.zeros(w.shape[0], self.nq, self.dk, dtype=w.dtype, device=w.device)
+            wide[:, :, :self.dv] = w.view(w.shape[0], self.nq, self.dv)
+            self.out_wide = wide.view(w.shape[0], self.nq * self.dk)
 
     def run(self, h, ctx, cache, layer, writes_cache=True):
         s, nt = self.spec, h.shape[0]
@@ -198,10 +221,23 @@ class NormedAttention(Part):
         kernels.qk_prepare(qkv, self.nq, self.nkv, self.dk, self.dv, float(s.eps),
                            self.w.get("q_norm.weight"), self.w.get("k_norm.weight"), angles, s.rot_dims,
                            mix, first, keep, meta.dest if writes_cache else None, kc, vc)
-        o = ctx.ws.take("attention.o", (nt, self.nq * self.dv), self.dtype)
-        kernels.attention_generic_dv(qkv, o, kc, vc, meta.block_table, ctx.cu_q, ctx.pos0, ctx.max_qlen,
-                                     self.nq, self.nkv, self.dk, self.dv, float(s.scale), s.window)
-        return linear_delta(o, self.w["out.weight"], ctx.ws, "attention.delta"), None
+        if not self._on_matrix_cores():
+            o = ctx.ws.take("attention.o", (nt, self.nq * self.dv), self.dtype)
+            kernels.attention_generic_dv(qkv, o, kc, vc, meta.block_table, ctx.cu_q, ctx.pos0, ctx.max_qlen,
+                                         self.nq, self.nkv, self.dk, self.dv, float(s.scale), s.window)
+            return linear_delta(o, self.w["out.weight"], ctx.ws, "attention.delta"), None
+        o = ctx.ws.take("attention.o", (nt, self.nq * self.dk), self.dtype)
+        planner = self.step_planner()
+        if ctx.all_single and planner is not None:
+            plan = meta.plans.get(planner, {})
+            kernels.attention_keys(qkv, o, kc, vc, meta.block_table, ctx.cu_q, ctx.pos0, ctx.max_kv_len,
+                                   self.nq, self.nkv, self.dk, float(s.scale), s.window,
+                                   units=plan.get("units"), seq_units=plan.get("seq_units"))
+        else:
+            kernels.attention_rows(qkv, o, kc, vc, meta.block_table, ctx.cu_q, ctx.pos0, ctx.max_qlen,
+                                   self.nq, self.nkv, self.dk, float(s.scale), s.window)
+        w = self.out_wide if self.out_wide is not None else self.w["out.weight"]
+        return linear_delta(o, w, ctx.ws, "attention.delta"), None
 
 
 register_part("attention_normed", NormedAttention)
