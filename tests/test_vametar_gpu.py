@@ -38,6 +38,11 @@ def _atol(dtype):
     return 2e-5 if dtype == "float32" else 2e-2
 
 
+def _rtol(dtype):
+    """One rounding of a result to the storage type, relative."""
+    return 1e-5 if dtype == "float32" else 2.0 ** -7
+
+
 # ----------------------------------------------------------------------------- mechanisms alone
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_token_shift_carries_the_last_row(dtype):
@@ -203,13 +208,13 @@ def test_attention_far_key_and_window_edges(where):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("geom", [(144, 3, 4), (48, 1, 1), (80, 5, 2), (640, 2, 3)])
+@pytest.mark.parametrize("geom", [(144, 3, 4), (48, 1, 1), (80, 5, 2), (640, 2, 3), (1600, 2, 2)])
 def test_diagonal_recurrence_pieces(dtype, geom):
     from transformer_amd import kernels as K
     C, nb, taps = geom
     td = torch.float32 if dtype == "float32" else torch.bfloat16
     rng = np.random.default_rng(5)
-    bs, lens = C // nb, [37, 1, 12]
+    bs, lens = C // nb, [200, 1, 70]     # more than one segment of the side-by-side scan
     w = {"y": np.zeros((C, 1)), "x": np.zeros((C, 1)), "y.b": 0.3 * rng.standard_normal(C),
          "x.b": 0.3 * rng.standard_normal(C), "conv": rng.standard_normal((C, taps)) / taps ** 0.5,
          "conv.b": 0.1 * rng.standard_normal(C), "ra": _bf(rng.standard_normal((nb, bs, bs)) / bs ** 0.5),
@@ -236,7 +241,7 @@ def test_diagonal_recurrence_pieces(dtype, geom):
     slots = _t([3, 0, 4], torch.int32)
     gw = _t(np.concatenate([w["ra"], w["ri"]]), td)
     gb = _t(np.concatenate([w["ra.b"], w["ri.b"]]))
-    for lo, hi in ((0, 1), (1, 3), (3, 40)):            # one token, two tokens, the rest
+    for lo, hi in ((0, 1), (1, 3), (3, 40), (40, 300)):     # one token, two tokens, portions
         part = [(y[lo:hi], x[lo:hi]) for y, x in seqs]
         keep = [i for i, p in enumerate(part) if len(p[0])]
         yx = _t(np.concatenate([np.concatenate(part[i], 1) for i in keep]), td)
@@ -246,12 +251,41 @@ def test_diagonal_recurrence_pieces(dtype, geom):
         K.rglru_gates(yx, C, _t(w["x.b"]), _t(w["conv"]), _t(w["conv.b"]), conv_state, gw, gb, _t(w["lam"]),
                       8.0, cu, sl, a, b)
         out = K.rglru_scan(yx, C, _t(w["y.b"]), _t(w["x.b"]), a, b, state, conv_state, cu, sl,
-                           torch.empty(nt, C, dtype=td, device=DEV))
+                           torch.empty(nt, C, dtype=td, device=DEV), max(len(part[i][0]) for i in keep),
+                           torch.empty(len(keep), C, device=DEV))
         got, at = out.float().cpu().numpy(), 0
         for i in keep:
             n = len(part[i][0])
-            np.testing.assert_allclose(got[at:at + n], want[i][lo:lo + n], atol=_atol(dtype))
+            np.testing.assert_allclose(got[at:at + n], want[i][lo:lo + n], atol=_atol(dtype), rtol=_rtol(dtype))
             at += n
+
+
+@pytest.mark.parametrize("geom", [(144, 3, 4), (512, 2, 2)])
+def test_recurrence_gates_of_long_steps_match_the_plain_kernel(geom):
+    """From 256 tokens on a bfloat16 step forms its gates through the library (u split into
+    two bfloat16 halves, float32 sums): the same decays and input terms as the 32-bit kernel."""
+    from transformer_amd import kernels as K
+    from transformer_amd.parts.linear import Workspace
+    C, nb, taps = geom
+    rng = np.random.default_rng(8)
+    bs, lens = C // nb, [290, 31]
+    nt = sum(lens)
+    yx = _t(rng.standard_normal((nt, 2 * C)) * 2, torch.bfloat16)
+    gw = _t(rng.standard_normal((2 * nb, bs, bs)) / bs ** 0.5, torch.bfloat16)
+    gb, xb, cb, lam = (_t(rng.standard_normal(n) * 0.3) for n in ((2 * nb, bs), C, C, C))
+    tp = _t(rng.standard_normal((C, taps)) / taps ** 0.5)
+    conv_state = _t(rng.standard_normal((3, taps - 1, C)))
+    cu, sl = _tables(lens), _t([2, 0], torch.int32)
+    out = []
+    for split in (False, True):
+        a, b = torch.empty(nt, C, device=DEV), torch.empty(nt, C, device=DEV)
+        if split:
+            K.rglru_gates_split(yx, C, xb, tp, cb, conv_state, gw, gb, lam, 8.0, cu, sl, a, b, Workspace(DEV))
+        else:
+            K.rglru_gates(yx, C, xb, tp, cb, conv_state, gw, gb, lam, 8.0, cu, sl, a, b)
+        out.append((a.cpu().numpy(), b.cpu().numpy()))
+    np.testing.assert_allclose(out[1][0], out[0][0], atol=2e-5)
+    np.testing.assert_allclose(out[1][1], out[0][1], atol=2e-4, rtol=1e-4)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -261,7 +295,7 @@ def test_gated_linear_attention_pieces(dtype, geom):
     H, dk, dv, rank = geom
     td = torch.float32 if dtype == "float32" else torch.bfloat16
     rng = np.random.default_rng(6)
-    tau, eps, lens = 4.0, 1e-5, [29, 1, 10]
+    tau, eps, lens = 4.0, 1e-5, [61, 1, 10]
     a2, a2b = _bf(rng.standard_normal((H * dk, rank))), rng.standard_normal(H * dk) + 2.0
     nw = 1 + 0.2 * rng.standard_normal(dv)
     width = 2 * H * dk + 2 * H * dv + rank
@@ -281,19 +315,21 @@ def test_gated_linear_attention_pieces(dtype, geom):
     want = [plain_one(s) for s in seqs]
     state = torch.zeros(4, H, dk, dv, device=DEV)
     slots = _t([1, 3, 0], torch.int32)
-    for lo, hi in ((0, 1), (1, 3), (3, 40)):
+    for lo, hi in ((0, 1), (1, 3), (3, 70)):
         part = [s[lo:hi] for s in seqs]
         keep = [i for i, p in enumerate(part) if len(p)]
         proj = _t(np.concatenate([part[i] for i in keep]), td)
         nt = proj.shape[0]
         cu, sl = _tables([len(part[i]) for i in keep]), slots[keep].contiguous()
         o = K.gla_recurrent(proj, H, dk, dv, rank, _t(a2, td), _t(a2b), tau, state, cu, sl,
-                            torch.empty(nt, H, dv, device=DEV))
+                            torch.empty(K.gla_row_parts(dk), nt, H, dv, device=DEV),
+                            torch.empty(nt, H * dk, device=DEV))
         out = K.gla_out(o, proj, H, dk, dv, _t(nw), eps, torch.empty(nt, H * dv, dtype=td, device=DEV))
         got, at = out.float().cpu().numpy(), 0
         for i in keep:
             n = len(part[i])
-            np.testing.assert_allclose(got[at:at + n], want[i][lo:lo + n], atol=1e-4 if dtype == "float32" else 3e-2)
+            np.testing.assert_allclose(got[at:at + n], want[i][lo:lo + n], atol=1e-4 if dtype == "float32" else 3e-2,
+                                       rtol=_rtol(dtype))
             at += n
 
 

@@ -24,6 +24,7 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
   T* row = qkv + (size_t)t * stride;
   const int nq = nh * dk, nk = nkv * dk, nv = nkv * dv;
   float sq = 0.f, sk = 0.f;
+#pragma unroll 8
   for (int i = threadIdx.x; i < nq + nk; i += 256) {
     const float v = to_f32(row[i]);
     buf[i] = v;
@@ -44,22 +45,25 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
   const int half = rot / 2;
   const float* ang = angles ? angles + (size_t)t * half * 2 : nullptr;
   const int page = dest ? dest[t] / TA_PAGE : 0, off = dest ? dest[t] % TA_PAGE : 0;
-  // every thread owns whole pairs, so nothing it reads is written by another thread
+  // Every thread reads the LDS copy and writes memory, so nothing it reads is written by another
+  // thread. All loads are unconditional (a coordinate that is not rotated reads angle 0 and is
+  // not changed by it), so that the loads of several turns are on their way together.
+  const float one = 1.f;
+#pragma unroll 4
   for (int i = threadIdx.x; i < nq + nk; i += 256) {
     const bool is_q = i < nq;
     const int j = is_q ? i : i - nq;
     const int head = j / dk, c = j - head * dk;
     const float f = is_q ? fq : fk;
-    const float* w = is_q ? wq : wk;
-    float v = buf[i] * f * (normed ? w[j] : 1.f);
-    if (ang && c < rot) {
-      const int pi = c < half ? c : c - half;
-      const float cs = ang[2 * pi], sn = ang[2 * pi + 1];
-      const int other = c < half ? i + half : i - half;
-      const int oj = c < half ? j + half : j - half;
-      const float o = buf[other] * f * (normed ? w[oj] : 1.f);
-      v = c < half ? v * cs - o * sn : v * cs + o * sn;
-    }
+    const float* w = normed ? (is_q ? wq : wk) : &one;
+    const bool turns = ang != nullptr && c < rot;
+    const int pi = turns ? (c < half ? c : c - half) : 0;
+    const int shift = turns ? (c < half ? half : -half) : 0;
+    const float cs = ang ? ang[2 * pi] : 1.f, sn = ang ? ang[2 * pi + 1] : 0.f;
+    const float wv = w[normed ? j : 0], wo = w[normed ? j + shift : 0];
+    float v = buf[i] * f * wv;
+    const float o = buf[i + shift] * f * wo;
+    if (turns) v = c < half ? v * cs - o * sn : v * cs + o * sn;
     if (is_q) {
       row[i] = from_f32<T>(v);
     } else if (dest) {

@@ -66,6 +66,60 @@ __global__ __launch_bounds__(256) void gated_add_rmsnorm_kernel(
     out[(size_t)i * d + c] = from_f32<TO>(row[c] * f * weight[c]);
 }
 
+// The same for rows whose length is a multiple of four and at most 4,096: 1,024 threads, four
+// columns each, everything a thread needs asked for at once (a row of a single-token step is
+// otherwise sixteen trips to memory, one after the other).
+template <typename TO>
+__global__ __launch_bounds__(1024) void gated_add_rmsnorm_wide_kernel(
+    float* __restrict__ x, const float* __restrict__ delta, int planes, size_t plane,
+    const float* __restrict__ delta_bias, const float* __restrict__ gate,
+    const float* __restrict__ gate_bias, float mult, const float* __restrict__ weight,
+    const int* __restrict__ rows, TO* __restrict__ out, int d, float eps, int store) {
+  __shared__ float red[16];
+  const int i = blockIdx.x;
+  const size_t r = rows ? (size_t)rows[i] : (size_t)i;
+  const int c = threadIdx.x * 4;
+  const bool on = c < d;
+  const size_t at = r * d + (on ? c : 0);
+  const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+  float4 v = *reinterpret_cast<const float4*>(x + at);
+  float4 w = *reinterpret_cast<const float4*>(weight + (on ? c : 0));
+  if (delta) {
+    float4 s = *reinterpret_cast<const float4*>(delta + at);
+    float4 g = gate ? *reinterpret_cast<const float4*>(gate + at) : zero;
+    const float4 gb = gate_bias ? *reinterpret_cast<const float4*>(gate_bias + (on ? c : 0)) : zero;
+    const float4 db = delta_bias ? *reinterpret_cast<const float4*>(delta_bias + (on ? c : 0)) : zero;
+    for (int p = 1; p < planes; ++p) {
+      const float4 e = *reinterpret_cast<const float4*>(delta + at + p * plane);
+      s.x += e.x; s.y += e.y; s.z += e.z; s.w += e.w;
+    }
+    s.x += db.x; s.y += db.y; s.z += db.z; s.w += db.w;
+    if (gate) {
+      s.x *= 1.0f / (1.0f + expf(-(g.x + gb.x)));
+      s.y *= 1.0f / (1.0f + expf(-(g.y + gb.y)));
+      s.z *= 1.0f / (1.0f + expf(-(g.z + gb.z)));
+      s.w *= 1.0f / (1.0f + expf(-(g.w + gb.w)));
+    }
+    v.x += mult * s.x; v.y += mult * s.y; v.z += mult * s.z; v.w += mult * s.w;
+    if (store && on) *reinterpret_cast<float4*>(x + at) = v;
+  }
+  float ss = on ? v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w : 0.f;
+  ss = wave_sum(ss);
+  if (threadIdx.x % TA_WAVE == 0) red[threadIdx.x / TA_WAVE] = ss;
+  __syncthreads();
+  float tot = 0.f;
+#pragma unroll
+  for (int k = 0; k < 16; ++k) tot += red[k];
+  const float f = rsqrtf(tot / (float)d + eps);
+  if (on) {
+    TO* o = out + (size_t)i * d + c;
+    o[0] = from_f32<TO>(v.x * f * w.x);
+    o[1] = from_f32<TO>(v.y * f * w.y);
+    o[2] = from_f32<TO>(v.z * f * w.z);
+    o[3] = from_f32<TO>(v.w * f * w.w);
+  }
+}
+
 extern "C" int ta_gated_add_rmsnorm(hipStream_t stream, int out_dtype, float* x, const float* delta,
                                     int planes, long long plane, const float* delta_bias,
                                     const float* gate, const float* gate_bias, float mult,
@@ -74,6 +128,17 @@ extern "C" int ta_gated_add_rmsnorm(hipStream_t stream, int out_dtype, float* x,
   TA_REQUIRE(n_out >= 0 && d > 0 && d <= 16000, "ta_gated_add_rmsnorm: bad sizes n=%d d=%d", n_out, d);
   TA_REQUIRE(planes >= 1 && planes <= TA_MAX_PLANES, "ta_gated_add_rmsnorm: %d planes", planes);
   if (n_out == 0) return 0;
+  const bool aligned = (((uintptr_t)x | (uintptr_t)delta | (uintptr_t)gate | (uintptr_t)gate_bias |
+                         (uintptr_t)delta_bias | (uintptr_t)weight | (uintptr_t)((size_t)plane * 4)) & 15) == 0;
+  if (d % 4 == 0 && d <= 4096 && aligned && (out_dtype == TA_F32 || out_dtype == TA_BF16)) {
+    if (out_dtype == TA_F32)
+      gated_add_rmsnorm_wide_kernel<float><<<n_out, 1024, 0, stream>>>(
+          x, delta, planes, (size_t)plane, delta_bias, gate, gate_bias, mult, weight, rows, (float*)out, d, eps, store);
+    else
+      gated_add_rmsnorm_wide_kernel<bf16_t><<<n_out, 1024, 0, stream>>>(
+          x, delta, planes, (size_t)plane, delta_bias, gate, gate_bias, mult, weight, rows, (bf16_t*)out, d, eps, store);
+    return ta_check_launch("ta_gated_add_rmsnorm");
+  }
   const size_t lds = (size_t)d * sizeof(float);
   if (out_dtype == TA_F32)
     gated_add_rmsnorm_kernel<float><<<n_out, 256, lds, stream>>>(
@@ -96,7 +161,7 @@ __global__ __launch_bounds__(256) void token_shift_kernel(
   const int b = seq_of_token(cu_q, batch, t);
   const int first = cu_q[b], last = cu_q[b + 1] - 1;
   float* st = state + (size_t)slots[b] * d;
-  for (int c = threadIdx.x; c < d; c += 256) {
+  for (int c = blockIdx.y * 256 + threadIdx.x; c < d; c += gridDim.y * 256) {
     const float cur = to_f32(h[(size_t)t * d + c]);
     float prev;
     if (t == first) {
@@ -113,10 +178,12 @@ __global__ __launch_bounds__(256) void token_shift_kernel(
 extern "C" int ta_token_shift(hipStream_t stream, int dtype, const void* h, void* hs, const float* mu,
                               float* state, const int* cu_q, const int* slots, int batch, int nt, int d) {
   TA_REQUIRE(batch > 0 && nt >= batch && d > 0, "ta_token_shift: bad sizes batch=%d nt=%d d=%d", batch, nt, d);
+  // few rows: a column tile per workgroup, so that a thread makes one trip to memory
+  dim3 g(nt, nt <= 256 ? (d + 255) / 256 : 1);
   if (dtype == TA_F32)
-    token_shift_kernel<float><<<nt, 256, 0, stream>>>((const float*)h, (float*)hs, mu, state, cu_q, slots, batch, d);
+    token_shift_kernel<float><<<g, 256, 0, stream>>>((const float*)h, (float*)hs, mu, state, cu_q, slots, batch, d);
   else if (dtype == TA_BF16)
-    token_shift_kernel<bf16_t><<<nt, 256, 0, stream>>>((const bf16_t*)h, (bf16_t*)hs, mu, state, cu_q, slots, batch, d);
+    token_shift_kernel<bf16_t><<<g, 256, 0, stream>>>((const bf16_t*)h, (bf16_t*)hs, mu, state, cu_q, slots, batch, d);
   else
     return ta_fail("ta_token_shift: unknown dtype %d", dtype);
   return ta_check_launch("ta_token_shift");

@@ -11,8 +11,8 @@
 // Gated linear attention ("gla"): per head a matrix state S [dk][dv]
 //     alpha_t = sigmoid(z_t)^(1/tau) per key channel, z_t = A2 (a1h_t) + bias
 //     S_t = diag(alpha_t) S_{t-1} + k_t v_t^T,  o_t = S_t^T q_t
-//   `gla_recurrent` walks a sequence's tokens in order with S in registers; `gla_out` applies the
-//   per-head RMS norm and the output gate.
+//   `gla_decay` forms alpha for all tokens at once, `gla_recurrent` walks a sequence's tokens in
+//   order with S in registers; `gla_out` applies the per-head RMS norm and the output gate.
 //
 // All state, decays, gates and sums are float32; tokens are walked in the same order however a
 // sequence was cut into steps, so the cut does not change a bit of the result.
@@ -110,6 +110,197 @@ __global__ __launch_bounds__(256) void rglru_gates_kernel(
   }
 }
 
+// The same with the gates' weights staged through LDS: a workgroup owns RGT_TT tokens x RGT_OC
+// output channels of one block and walks the block's inputs in turns of RGT_KC, each turn's
+// weights loaded row by row in whole pieces and laid down transposed, so that a thread reads its
+// channel's weight and a wave shares every u. Used whenever a block's inputs fit the LDS.
+#define RGT_TT 16
+#define RGT_OC 64
+#define RGT_KC 32
+
+template <typename T, typename TW>
+__global__ __launch_bounds__(256) void rglru_gates_tiled_kernel(
+    const T* __restrict__ yx, int stride, int xoff, const float* __restrict__ xbias,
+    const float* __restrict__ taps, const float* __restrict__ conv_bias, int K,
+    const float* __restrict__ conv_state, const TW* __restrict__ gates_w,
+    const float* __restrict__ gates_b, const float* __restrict__ lam, float c0,
+    const int* __restrict__ cu_q, const int* __restrict__ slots, int batch, int nt, int C, int nb,
+    int bsp, float* __restrict__ a_out, float* __restrict__ b_out) {
+  extern __shared__ float sm[];
+  float* u = sm;                               // [RGT_TT][bsp], zero beyond bs
+  float* wrs = u + RGT_TT * bsp;               // [RGT_KC][RGT_OC]
+  float* wis = wrs + RGT_KC * RGT_OC;
+  __shared__ int s_start[RGT_TT], s_slot[RGT_TT];
+  const int bs = C / nb;
+  const int tiles = (bs + RGT_OC - 1) / RGT_OC;
+  const int blk = blockIdx.y / tiles, o0 = (blockIdx.y % tiles) * RGT_OC;
+  const int t0 = blockIdx.x * RGT_TT;
+  if (threadIdx.x < RGT_TT) {
+    const int t = t0 + threadIdx.x;
+    int st = 0, sl = 0;
+    if (t < nt) {
+      const int b = seq_of_token_r(cu_q, batch, t);
+      st = cu_q[b];
+      sl = slots[b];
+    }
+    s_start[threadIdx.x] = st;
+    s_slot[threadIdx.x] = sl;
+  }
+  __syncthreads();
+#pragma unroll 4
+  for (int idx = threadIdx.x; idx < RGT_TT * bsp; idx += 256) {
+    const int tt = idx / bsp, cc = idx - tt * bsp;
+    const int t = t0 + tt, c = blk * bs + cc;
+    // both places a tap may read (this step's rows, the sequence's memory) are asked for
+    // whatever the case, at addresses that exist, and one is chosen: no load waits for a branch
+    const bool on = t < nt && cc < bs;
+    const int ts = on ? t : 0, cz = on ? c : 0;
+    const int start = s_start[tt];
+    const float* cs = conv_state + ((size_t)s_slot[tt] * (K - 1)) * C;
+    const float xb = xbias[cz];
+    float acc = conv_bias[cz];
+    for (int j = 0; j < K; ++j) {
+      const int tp = ts - (K - 1 - j);
+      const bool here = tp >= start;
+      const float a = to_f32(yx[(size_t)(here ? tp : ts) * stride + xoff + cz]) + xb;
+      const float m = K > 1 ? cs[(size_t)(here ? 0 : K - 1 + (tp - start)) * C + cz] : 0.f;
+      acc = fmaf(taps[(size_t)cz * K + j], here ? a : m, acc);
+    }
+    u[idx] = on ? acc : 0.f;
+  }
+  const int o = threadIdx.x % RGT_OC, tg = threadIdx.x / RGT_OC;      // tokens tg*4 .. tg*4+3
+  const int lr = threadIdx.x / 4, lseg = (threadIdx.x % 4) * 8;       // staging: row lr, 8 inputs from lseg
+  float ar[4] = {0.f, 0.f, 0.f, 0.f}, ai[4] = {0.f, 0.f, 0.f, 0.f};
+  const bool row_ok = o0 + lr < bs;
+  const TW* wr = gates_w + ((size_t)blk * bs + (row_ok ? o0 + lr : 0)) * bs;
+  const TW* wi = gates_w + ((size_t)(nb + blk) * bs + (row_ok ? o0 + lr : 0)) * bs;
+  float nr[8], ni[8];                           // the next turn's weights, on their way
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int in = k0 + lseg + e;
+      const bool ok = row_ok && in < bs;
+      const float a = to_f32(wr[ok ? in : 0]), b = to_f32(wi[ok ? in : 0]);
+      nr[e] = ok ? a : 0.f;
+      ni[e] = ok ? b : 0.f;
+    }
+  };
+  fetch(0);
+  for (int k0 = 0; k0 < bs; k0 += RGT_KC) {
+    __syncthreads();                            // u is complete / the last turn's weights are used up
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      wrs[(lseg + e) * RGT_OC + lr] = nr[e];
+      wis[(lseg + e) * RGT_OC + lr] = ni[e];
+    }
+    __syncthreads();
+    if (k0 + RGT_KC < bs) fetch(k0 + RGT_KC);
+    const float* ub = u + (tg * 4) * bsp + k0;
+#pragma unroll 8
+    for (int in = 0; in < RGT_KC; ++in) {
+      const float a = wrs[in * RGT_OC + o], b = wis[in * RGT_OC + o];
+#pragma unroll
+      for (int tk = 0; tk < 4; ++tk) {
+        const float uu = ub[tk * bsp + in];
+        ar[tk] = fmaf(a, uu, ar[tk]);
+        ai[tk] = fmaf(b, uu, ai[tk]);
+      }
+    }
+  }
+  if (o0 + o < bs) {
+    const int c = blk * bs + o0 + o;
+    const float br = gates_b[(size_t)blk * bs + o0 + o], bi = gates_b[(size_t)(nb + blk) * bs + o0 + o];
+    const float sp = softplusf_(lam[c]);
+#pragma unroll
+    for (int tk = 0; tk < 4; ++tk) {
+      const int tt = tg * 4 + tk, t = t0 + tt;
+      if (t < nt) {
+        const float r = sigmoidf_(ar[tk] + br), g = sigmoidf_(ai[tk] + bi);
+        const float loga = -c0 * r * sp;
+        a_out[(size_t)t * C + c] = expf(loga);
+        b_out[(size_t)t * C + c] = sqrtf(-expm1f(2.0f * loga)) * g * u[tt * bsp + o0 + o];
+      }
+    }
+  }
+}
+
+// Long steps of a bfloat16 engine take the gates' block-diagonal products to the matrix cores
+// without giving up 32-bit inputs: `rglru_conv_split` leaves u in float32 and as two bfloat16
+// numbers hi + lo = u (to 16 bits of mantissa), the library multiplies both by the bfloat16
+// weights with float32 sums, and `rglru_gates_finish` adds the two products and forms a_t and
+// the input term exactly as the kernels above do.
+template <typename T>
+__global__ __launch_bounds__(256) void rglru_conv_split_kernel(
+    const T* __restrict__ yx, int stride, int xoff, const float* __restrict__ xbias,
+    const float* __restrict__ taps, const float* __restrict__ conv_bias, int K,
+    const float* __restrict__ conv_state, const int* __restrict__ cu_q, const int* __restrict__ slots,
+    int batch, int nt, int C, float* __restrict__ u_out, bf16_t* __restrict__ hi, bf16_t* __restrict__ lo) {
+  const int t = blockIdx.y;
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= C) return;
+  const int b = seq_of_token_r(cu_q, batch, t);
+  const int start = cu_q[b];
+  const float* cs = conv_state + ((size_t)slots[b] * (K - 1)) * C;
+  float acc = conv_bias[c];
+  for (int j = 0; j < K; ++j) {
+    const int tp = t - (K - 1 - j);
+    float xin;
+    if (tp >= start) xin = to_f32(yx[(size_t)tp * stride + xoff + c]) + xbias[c];
+    else xin = cs[(size_t)(K - 1 + (tp - start)) * C + c];
+    acc = fmaf(taps[(size_t)c * K + j], xin, acc);
+  }
+  const size_t at = (size_t)t * C + c;
+  u_out[at] = acc;
+  const bf16_t h = from_f32<bf16_t>(acc);
+  hi[at] = h;
+  lo[at] = from_f32<bf16_t>(acc - to_f32(h));
+}
+
+__global__ __launch_bounds__(256) void rglru_gates_finish_kernel(
+    const float* __restrict__ g, const float* __restrict__ u, const float* __restrict__ gates_b,
+    const float* __restrict__ lam, float c0, int nt, int C, int nb, float* __restrict__ a_out,
+    float* __restrict__ b_out) {
+  // g: [2 gates][nb][2 halves * nt][bs]: the products of hi (rows 0..nt) and lo (rows nt..2nt)
+  const int t = blockIdx.y;
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= C) return;
+  const int bs = C / nb, blk = c / bs, cc = c - blk * bs;
+  const size_t gate = (size_t)nb * 2 * nt * bs;
+  const size_t at = ((size_t)blk * 2 * nt + t) * bs + cc, half = (size_t)nt * bs;
+  const float zr = (g[at] + g[at + half]) + gates_b[(size_t)blk * bs + cc];
+  const float zi = (g[gate + at] + g[gate + at + half]) + gates_b[(size_t)(nb + blk) * bs + cc];
+  const float r = sigmoidf_(zr), gi = sigmoidf_(zi);
+  const float loga = -c0 * r * softplusf_(lam[c]);
+  a_out[(size_t)t * C + c] = expf(loga);
+  b_out[(size_t)t * C + c] = sqrtf(-expm1f(2.0f * loga)) * gi * u[(size_t)t * C + c];
+}
+
+extern "C" int ta_rglru_conv_split(hipStream_t stream, int dtype, const void* yx, int stride, int xoff,
+                                   const float* xbias, const float* taps, const float* conv_bias, int K,
+                                   const float* conv_state, const int* cu_q, const int* slots, int batch,
+                                   int nt, int C, float* u_out, void* hi, void* lo) {
+  TA_REQUIRE(batch > 0 && nt >= batch && nt <= 65535 && C > 0 && K >= 1, "ta_rglru_conv_split: bad sizes");
+  dim3 g((C + 255) / 256, nt);
+  if (dtype == TA_F32)
+    rglru_conv_split_kernel<float><<<g, 256, 0, stream>>>((const float*)yx, stride, xoff, xbias, taps, conv_bias, K,
+        conv_state, cu_q, slots, batch, nt, C, u_out, (bf16_t*)hi, (bf16_t*)lo);
+  else if (dtype == TA_BF16)
+    rglru_conv_split_kernel<bf16_t><<<g, 256, 0, stream>>>((const bf16_t*)yx, stride, xoff, xbias, taps, conv_bias, K,
+        conv_state, cu_q, slots, batch, nt, C, u_out, (bf16_t*)hi, (bf16_t*)lo);
+  else
+    return ta_fail("ta_rglru_conv_split: unknown dtype %d", dtype);
+  return ta_check_launch("ta_rglru_conv_split");
+}
+
+extern "C" int ta_rglru_gates_finish(hipStream_t stream, const float* g, const float* u, const float* gates_b,
+                                     const float* lam, float c0, int nt, int C, int nb, float* a_out,
+                                     float* b_out) {
+  TA_REQUIRE(nt > 0 && nt <= 65535 && C > 0 && nb > 0 && C % nb == 0, "ta_rglru_gates_finish: bad sizes");
+  dim3 gr((C + 255) / 256, nt);
+  rglru_gates_finish_kernel<<<gr, 256, 0, stream>>>(g, u, gates_b, lam, c0, nt, C, nb, a_out, b_out);
+  return ta_check_launch("ta_rglru_gates_finish");
+}
+
 // yx: [nt, stride] rows holding the y branch at column 0 and the x branch at column xoff (C each);
 // xbias [C]; taps [C, K]; conv_state [slots, K-1, C] float32 (inputs of the last K-1 tokens);
 // gates_w [2*nb, bs, bs] (recurrence gate blocks, then input gate blocks), gates_b [2*nb, bs];
@@ -123,6 +314,21 @@ extern "C" int ta_rglru_gates(hipStream_t stream, int dtype, int wdtype, const v
              "ta_rglru_gates: bad sizes nt=%d C=%d blocks=%d taps=%d", nt, C, nb, K);
   TA_REQUIRE(nb <= 65535, "ta_rglru_gates: too many blocks");
   const int bs = C / nb;
+  const int bsp = (bs + RGT_KC - 1) / RGT_KC * RGT_KC;
+  const size_t lds_tiled = ((size_t)RGT_TT * bsp + 2 * RGT_KC * RGT_OC) * sizeof(float);
+  const int tiles = (bs + RGT_OC - 1) / RGT_OC;
+  if (lds_tiled <= 64000 && (long long)nb * tiles <= 65535) {
+    dim3 gt((nt + RGT_TT - 1) / RGT_TT, nb * tiles);
+#define RGT_LAUNCH(T, TW)                                                                              \
+  rglru_gates_tiled_kernel<T, TW><<<gt, 256, lds_tiled, stream>>>((const T*)yx, stride, xoff, xbias, taps, conv_bias, K, \
+      conv_state, (const TW*)gates_w, gates_b, lam, c0, cu_q, slots, batch, nt, C, nb, bsp, a_out, b_out)
+    if (dtype == TA_F32 && wdtype == TA_F32) RGT_LAUNCH(float, float);
+    else if (dtype == TA_BF16 && wdtype == TA_BF16) RGT_LAUNCH(bf16_t, bf16_t);
+    else if (dtype == TA_BF16 && wdtype == TA_F32) RGT_LAUNCH(bf16_t, float);
+    else return ta_fail("ta_rglru_gates: unsupported dtypes %d / %d", dtype, wdtype);
+#undef RGT_LAUNCH
+    return ta_check_launch("ta_rglru_gates");
+  }
   const size_t lds = (size_t)RG_TT * bs * sizeof(float);
   TA_REQUIRE(lds <= 60000, "ta_rglru_gates: blocks of %d channels do not fit", bs);
   dim3 g((nt + RG_TT - 1) / RG_TT, nb);
@@ -184,189 +390,363 @@ __global__ __launch_bounds__(256) void rglru_scan_kernel(
   }
 }
 
-// state [slots, C] float32; out [nt, C]. Runs after ta_rglru_gates of the same step.
+// ------------------------------------------------------------------ rglru: scan of long steps
+// A step that brings many tokens per sequence is cut into segments of RG_SEG tokens that are
+// scanned side by side: `rglru_local_kernel` scans each segment from S = 0 and leaves, in place
+// of (a_t, b_t), the product of the decays since the segment's start and the locally scanned
+// value; `rglru_apply_kernel` forms the state at its segment's start from the segments in front
+// of it (S' = P_last S + local_last, in order) and finishes S_t = local_t + P_t S_start.
+#define RG_SEG 64
+
+__global__ __launch_bounds__(256) void rglru_local_kernel(float* __restrict__ a_io, float* __restrict__ b_io,
+                                                          const float* __restrict__ state, float* __restrict__ s0,
+                                                          const int* __restrict__ cu_q,
+                                                          const int* __restrict__ slots, int C) {
+  const int b = blockIdx.z, seg = blockIdx.y;
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  const int start = cu_q[b] + seg * RG_SEG, end = min(cu_q[b + 1], start + RG_SEG);
+  if (c >= C || start >= end) return;
+  // the state as the step found it, for every segment's workgroup of the next kernel (whose
+  // last segment overwrites the state itself)
+  if (seg == 0) s0[(size_t)b * C + c] = state[(size_t)slots[b] * C + c];
+  float S = 0.f, P = 1.f;
+  int t = start;
+  for (; t + 8 <= end; t += 8) {
+    float a[8], bb[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      a[i] = a_io[(size_t)(t + i) * C + c];
+      bb[i] = b_io[(size_t)(t + i) * C + c];
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      S = fmaf(a[i], S, bb[i]);
+      P *= a[i];
+      a_io[(size_t)(t + i) * C + c] = P;
+      b_io[(size_t)(t + i) * C + c] = S;
+    }
+  }
+  for (; t < end; ++t) {
+    S = fmaf(a_io[(size_t)t * C + c], S, b_io[(size_t)t * C + c]);
+    P *= a_io[(size_t)t * C + c];
+    a_io[(size_t)t * C + c] = P;
+    b_io[(size_t)t * C + c] = S;
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void rglru_apply_kernel(
+    const T* __restrict__ yx, int stride, int xoff, const float* __restrict__ ybias,
+    const float* __restrict__ xbias, const float* __restrict__ p_in, const float* __restrict__ l_in,
+    const float* __restrict__ s0, float* __restrict__ state, float* __restrict__ conv_state, int K,
+    const int* __restrict__ cu_q,
+    const int* __restrict__ slots, int C, T* __restrict__ out) {
+  const int b = blockIdx.z, seg = blockIdx.y;
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  const int first = cu_q[b], last = cu_q[b + 1];
+  const int start = first + seg * RG_SEG, end = min(last, start + RG_SEG);
+  if (c >= C || start >= end) return;
+  const size_t slot = (size_t)slots[b];
+  float S0 = s0[(size_t)b * C + c];
+  for (int s = 0; s < seg; ++s) {              // the segments in front, in order
+    const size_t e = (size_t)(first + (s + 1) * RG_SEG - 1) * C + c;
+    S0 = fmaf(p_in[e], S0, l_in[e]);
+  }
+  const float yb = ybias[c];
+  float S = S0;
+  for (int t = start; t < end; ++t) {
+    S = fmaf(p_in[(size_t)t * C + c], S0, l_in[(size_t)t * C + c]);
+    out[(size_t)t * C + c] = from_f32<T>(S * gelu_tanhf_(to_f32(yx[(size_t)t * stride + c]) + yb));
+  }
+  if (end != last) return;
+  // the sequence's last segment leaves the state and the convolution's memory
+  state[slot * C + c] = S;
+  const int n = last - first;
+  float* cs = conv_state + slot * (size_t)(K - 1) * C;
+  const float xb = xbias[c];
+  for (int j = 0; j < K - 1; ++j) {
+    const int src = j + n;
+    float v;
+    if (src < K - 1) v = cs[(size_t)src * C + c];
+    else v = to_f32(yx[(size_t)(first + src - (K - 1)) * stride + xoff + c]) + xb;
+    cs[(size_t)j * C + c] = v;
+  }
+}
+
+// state [slots, C] float32; out [nt, C]. Runs after ta_rglru_gates of the same step. a_io, b_io
+// [nt, C]: what ta_rglru_gates left; overwritten when the step is long (max_qlen > RG_SEG: the
+// segments are then scanned side by side, and s0 [batch, C] float32 is scratch for that).
 extern "C" int ta_rglru_scan(hipStream_t stream, int dtype, const void* yx, int stride, int xoff,
-                             const float* ybias, const float* xbias, const float* a_in, const float* b_in,
+                             const float* ybias, const float* xbias, float* a_io, float* b_io,
                              float* state, float* conv_state, int K, const int* cu_q, const int* slots,
-                             int batch, int C, void* out) {
-  TA_REQUIRE(batch > 0 && batch <= 65535 && C > 0 && K >= 1, "ta_rglru_scan: bad sizes");
+                             int batch, int max_qlen, int C, float* s0, void* out) {
+  TA_REQUIRE(batch > 0 && batch <= 65535 && C > 0 && K >= 1 && max_qlen >= 1, "ta_rglru_scan: bad sizes");
+  if (max_qlen > RG_SEG) {
+    const int segs = (max_qlen + RG_SEG - 1) / RG_SEG;
+    TA_REQUIRE(segs <= 65535 && s0 != nullptr, "ta_rglru_scan: step too long, or no scratch");
+    dim3 g((C + 255) / 256, segs, batch);
+    rglru_local_kernel<<<g, 256, 0, stream>>>(a_io, b_io, state, s0, cu_q, slots, C);
+    if (dtype == TA_F32)
+      rglru_apply_kernel<float><<<g, 256, 0, stream>>>((const float*)yx, stride, xoff, ybias, xbias, a_io, b_io, s0,
+                                                      state, conv_state, K, cu_q, slots, C, (float*)out);
+    else if (dtype == TA_BF16)
+      rglru_apply_kernel<bf16_t><<<g, 256, 0, stream>>>((const bf16_t*)yx, stride, xoff, ybias, xbias, a_io, b_io, s0,
+                                                       state, conv_state, K, cu_q, slots, C, (bf16_t*)out);
+    else
+      return ta_fail("ta_rglru_scan: unknown dtype %d", dtype);
+    return ta_check_launch("ta_rglru_scan");
+  }
   dim3 g((C + 255) / 256, batch);
   if (dtype == TA_F32)
-    rglru_scan_kernel<float><<<g, 256, 0, stream>>>((const float*)yx, stride, xoff, ybias, xbias, a_in, b_in, state,
+    rglru_scan_kernel<float><<<g, 256, 0, stream>>>((const float*)yx, stride, xoff, ybias, xbias, a_io, b_io, state,
                                                    conv_state, K, cu_q, slots, C, (float*)out);
   else if (dtype == TA_BF16)
-    rglru_scan_kernel<bf16_t><<<g, 256, 0, stream>>>((const bf16_t*)yx, stride, xoff, ybias, xbias, a_in, b_in, state,
+    rglru_scan_kernel<bf16_t><<<g, 256, 0, stream>>>((const bf16_t*)yx, stride, xoff, ybias, xbias, a_io, b_io, state,
                                                     conv_state, K, cu_q, slots, C, (bf16_t*)out);
   else
     return ta_fail("ta_rglru_scan: unknown dtype %d", dtype);
   return ta_check_launch("ta_rglru_scan");
 }
 
-// ------------------------------------------------------------------ gla: recurrence
-#define GLA_TC 8      // tokens whose operands are staged together
-
-template <typename T, typename TW, int R>
-__global__ __launch_bounds__(256) void gla_recurrent_kernel(
-    const T* __restrict__ proj, int stride, int qoff, int koff, int voff, int aoff, int rank,
-    const TW* __restrict__ a2, const float* __restrict__ a2b, float inv_tau, float qscale,
-    float* __restrict__ state, const int* __restrict__ cu_q, const int* __restrict__ slots,
-    int H, int dk, int dv, int CT, int P, float* __restrict__ o_out) {
-  extern __shared__ float sm[];
-  const int PR = P * R;                    // padded key width
-  float* sq = sm;                          // [TC][PR]
-  float* sk = sq + GLA_TC * PR;            // [TC][PR]
-  float* sa = sk + GLA_TC * PR;            // [TC][PR]
-  float* sv = sa + GLA_TC * PR;            // [TC][CT]
-  float* s1 = sv + GLA_TC * CT;            // [TC][rank]
-  float* part = s1 + GLA_TC * rank;        // [TC][P][CT]
-  const int b = blockIdx.x, h = blockIdx.y, col0 = blockIdx.z * CT;
-  const int start = cu_q[b], end = cu_q[b + 1];
-  const size_t slot = (size_t)slots[b];
-  const int j = threadIdx.x % CT, p = threadIdx.x / CT;
-  const bool active = p < P && col0 + j < dv;
-  float* st = state + ((slot * H + h) * dk) * (size_t)dv;
-  float S[R];
-#pragma unroll
-  for (int r = 0; r < R; ++r) {
-    const int i = p * R + r;
-    S[r] = (active && i < dk) ? st[(size_t)i * dv + col0 + j] : 0.f;
-  }
-  for (int t0 = start; t0 < end; t0 += GLA_TC) {
-    const int n = end - t0 < GLA_TC ? end - t0 : GLA_TC;
-    for (int idx = threadIdx.x; idx < GLA_TC * PR; idx += 256) {
-      const int tt = idx / PR, i = idx - tt * PR;
-      float qv = 0.f, kv = 0.f;
-      if (tt < n && i < dk) {
-        const T* row = proj + (size_t)(t0 + tt) * stride;
-        qv = to_f32(row[qoff + h * dk + i]) * qscale;
-        kv = to_f32(row[koff + h * dk + i]);
-      }
-      sq[idx] = qv;
-      sk[idx] = kv;
-    }
-    for (int idx = threadIdx.x; idx < GLA_TC * CT; idx += 256) {
-      const int tt = idx / CT, c = idx - tt * CT;
-      sv[idx] = (tt < n && col0 + c < dv) ? to_f32(proj[(size_t)(t0 + tt) * stride + voff + h * dv + col0 + c]) : 0.f;
-    }
-    for (int idx = threadIdx.x; idx < GLA_TC * rank; idx += 256) {
-      const int tt = idx / rank, r = idx - tt * rank;
-      s1[idx] = tt < n ? to_f32(proj[(size_t)(t0 + tt) * stride + aoff + r]) : 0.f;
-    }
-    __syncthreads();
-    for (int idx = threadIdx.x; idx < GLA_TC * PR; idx += 256) {
-      const int tt = idx / PR, i = idx - tt * PR;
-      float al = 0.f;
-      if (tt < n && i < dk) {
-        const TW* w = a2 + (size_t)(h * dk + i) * rank;
-        float z = a2b[h * dk + i];
-        for (int r = 0; r < rank; ++r) z = fmaf(to_f32(w[r]), s1[tt * rank + r], z);
-        // log sigmoid(z) = min(z, 0) - log1p(exp(-|z|))
-        al = expf((fminf(z, 0.f) - log1pf(expf(-fabsf(z)))) * inv_tau);
-      }
-      sa[idx] = al;
-    }
-    __syncthreads();
-    if (active) {
-      for (int tt = 0; tt < n; ++tt) {
-        const float vj = sv[tt * CT + j];
-        const float* qa = sq + tt * PR + p * R;
-        const float* ka = sk + tt * PR + p * R;
-        const float* aa = sa + tt * PR + p * R;
-        float po = 0.f;
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-          S[r] = fmaf(aa[r], S[r], ka[r] * vj);
-          po = fmaf(S[r], qa[r], po);
-        }
-        part[(tt * P + p) * CT + j] = po;
-      }
-    }
-    __syncthreads();
-    for (int idx = threadIdx.x; idx < n * CT; idx += 256) {
-      const int tt = idx / CT, c = idx - tt * CT;
-      if (col0 + c < dv) {
-        float o = 0.f;
-        for (int pp = 0; pp < P; ++pp) o += part[(tt * P + pp) * CT + c];
-        o_out[((size_t)(t0 + tt) * H + h) * dv + col0 + c] = o;
-      }
-    }
-    // the next turn's loads touch sq/sk/sv/s1 only; `part` is rewritten after two barriers
-  }
-  if (active) {
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-      const int i = p * R + r;
-      if (i < dk) st[(size_t)i * dv + col0 + j] = S[r];
-    }
+// ------------------------------------------------------------------ gla: decay per key channel
+template <typename T, typename TW>
+__global__ __launch_bounds__(256) void gla_decay_kernel(const T* __restrict__ proj, int stride, int aoff, int rank,
+                                                        const TW* __restrict__ a2, const float* __restrict__ a2b,
+                                                        float inv_tau, int n, float* __restrict__ alpha) {
+  extern __shared__ float low[];          // [rank]
+  const size_t t = blockIdx.x;
+  for (int r = threadIdx.x; r < rank; r += 256) low[r] = to_f32(proj[t * stride + aoff + r]);
+  __syncthreads();
+  for (int c = blockIdx.y * 256 + threadIdx.x; c < n; c += gridDim.y * 256) {
+    const TW* w = a2 + (size_t)c * rank;
+    float z = a2b[c];
+    for (int r = 0; r < rank; ++r) z = fmaf(to_f32(w[r]), low[r], z);
+    // sigmoid(z)^(1/tau) = exp(log sigmoid(z) / tau), log sigmoid(z) = min(z, 0) - log1p(exp(-|z|))
+    alpha[t * n + c] = expf((fminf(z, 0.f) - log1pf(expf(-fabsf(z)))) * inv_tau);
   }
 }
 
+// ------------------------------------------------------------------ gla: recurrence
+// A workgroup owns GLA_RT key channels x GLA_CT value columns of one (sequence, head); a thread
+// keeps 4 x 2 entries of S in registers, so every operand it reads from LDS feeds two or four
+// multiply-adds. A chunk's operands are staged in LDS while the next chunk's are already on
+// their way from memory. The readout q.S is summed over a workgroup's rows here and over the
+// workgroups that share a head's columns by `gla_out` (o_out holds one plane per group of
+// GLA_RT key channels).
+// GLA_TC tokens are staged together: 32 for prompts, 8 for steps of few tokens per sequence
+// (a chunk always costs all of its turns)
+#define GLA_RT 32     // key channels per workgroup
+#define GLA_CT 64     // value columns per workgroup
+
+template <int GLA_TC>
+struct GlaOperands {  // what one thread brings in for a chunk
+  float q[GLA_TC * GLA_RT / 256], k[GLA_TC * GLA_RT / 256], a[GLA_TC * GLA_RT / 256], v[GLA_TC * GLA_CT / 256];
+};
+
+template <typename T, int GLA_TC>
+__global__ __launch_bounds__(256) void gla_recurrent_kernel(
+    const T* __restrict__ proj, int stride, int qoff, int koff, int voff, const float* __restrict__ alpha,
+    float qscale, float* __restrict__ state, const int* __restrict__ cu_q, const int* __restrict__ slots,
+    int H, int dk, int dv, int col_tiles, size_t plane, float* __restrict__ o_out) {
+  __shared__ float sq[GLA_TC][GLA_RT], sk[GLA_TC][GLA_RT], sa[GLA_TC][GLA_RT];
+  __shared__ float sv[GLA_TC][GLA_CT];
+  __shared__ float part[GLA_TC][4][GLA_CT];
+  constexpr int NQ = GLA_TC * GLA_RT / 256, NV = GLA_TC * GLA_CT / 256;
+  const int b = blockIdx.x, h = blockIdx.y;
+  const int rpart = blockIdx.z / col_tiles, ctile = blockIdx.z % col_tiles;
+  const int row0 = rpart * GLA_RT, col0 = ctile * GLA_CT;
+  const int start = cu_q[b], end = cu_q[b + 1];
+  const size_t slot = (size_t)slots[b];
+  const int tid = threadIdx.x;
+  const int rg = tid / 32, cg = tid % 32;          // rows rg*4.., columns cg*2..
+  float* st = state + ((slot * H + h) * dk) * (size_t)dv;
+  float S[4][2];
+#pragma unroll
+  for (int r = 0; r < 4; ++r)
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      const int i = row0 + rg * 4 + r, j = col0 + cg * 2 + c;
+      S[r][c] = (i < dk && j < dv) ? st[(size_t)i * dv + j] : 0.f;
+    }
+  // Loads are asked for two chunks ahead (a trip to memory takes longer than a chunk's
+  // arithmetic); a position that is not there reads a harmless address and is replaced.
+  auto fetch = [&](GlaOperands<GLA_TC>& o, int t0) {
+#pragma unroll
+    for (int e = 0; e < NQ; ++e) {
+      const int idx = tid + 256 * e, tt = idx / GLA_RT, i = row0 + idx % GLA_RT;
+      const bool ok = t0 + tt < end && i < dk;
+      const size_t row = (size_t)(ok ? t0 + tt : start);
+      const int ii = ok ? i : 0;
+      const float qv = to_f32(proj[row * stride + qoff + h * dk + ii]);
+      const float kv = to_f32(proj[row * stride + koff + h * dk + ii]);
+      const float av = alpha[row * ((size_t)H * dk) + h * dk + ii];
+      o.q[e] = ok ? qv * qscale : 0.f;
+      o.k[e] = ok ? kv : 0.f;
+      o.a[e] = ok ? av : 1.f;           // a token that is not there leaves S as it is
+    }
+#pragma unroll
+    for (int e = 0; e < NV; ++e) {
+      const int idx = tid + 256 * e, tt = idx / GLA_CT, j = col0 + idx % GLA_CT;
+      const bool ok = t0 + tt < end && j < dv;
+      const float vv = to_f32(proj[(size_t)(ok ? t0 + tt : start) * stride + voff + h * dv + (ok ? j : 0)]);
+      o.v[e] = ok ? vv : 0.f;
+    }
+  };
+  auto turn = [&](GlaOperands<GLA_TC>& o, int t0) {
+    const int n = end - t0 < GLA_TC ? end - t0 : GLA_TC;
+#pragma unroll
+    for (int e = 0; e < NQ; ++e) {
+      const int idx = tid + 256 * e;
+      (&sq[0][0])[idx] = o.q[e];
+      (&sk[0][0])[idx] = o.k[e];
+      (&sa[0][0])[idx] = o.a[e];
+    }
+#pragma unroll
+    for (int e = 0; e < NV; ++e) (&sv[0][0])[tid + 256 * e] = o.v[e];
+    __syncthreads();
+    if (t0 + 2 * GLA_TC < end) fetch(o, t0 + 2 * GLA_TC);
+    // all GLA_TC tokens always (those past the end carry k = 0, alpha = 1), in groups of eight
+    // whose count is fixed: the compiler asks for the next tokens' operands while it works on
+    // this one, and the readouts stay in registers until the group is done, so only the update
+    // of S itself is a chain.
+#pragma unroll 1
+    for (int g0 = 0; g0 < GLA_TC; g0 += 8) {
+      float p0[8], p1[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int tt = g0 + u;
+        const float4 q4 = *reinterpret_cast<const float4*>(&sq[tt][rg * 4]);
+        const float4 k4 = *reinterpret_cast<const float4*>(&sk[tt][rg * 4]);
+        const float4 a4 = *reinterpret_cast<const float4*>(&sa[tt][rg * 4]);
+        const float2 v2 = *reinterpret_cast<const float2*>(&sv[tt][cg * 2]);
+        const float qs[4] = {q4.x, q4.y, q4.z, q4.w}, ks[4] = {k4.x, k4.y, k4.z, k4.w};
+        const float as[4] = {a4.x, a4.y, a4.z, a4.w};
+        float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          S[r][0] = fmaf(as[r], S[r][0], ks[r] * v2.x);
+          S[r][1] = fmaf(as[r], S[r][1], ks[r] * v2.y);
+          a0 = fmaf(S[r][0], qs[r], a0);
+          a1 = fmaf(S[r][1], qs[r], a1);
+        }
+        p0[u] = a0;
+        p1[u] = a1;
+      }
+      // the two row groups of a wave, then the four waves through LDS
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const float a0 = p0[u] + __shfl_xor(p0[u], 32, TA_WAVE);
+        const float a1 = p1[u] + __shfl_xor(p1[u], 32, TA_WAVE);
+        if ((tid & 32) == 0) {
+          part[g0 + u][tid / 64][cg * 2] = a0;
+          part[g0 + u][tid / 64][cg * 2 + 1] = a1;
+        }
+      }
+    }
+    __syncthreads();
+    for (int idx = tid; idx < n * GLA_CT; idx += 256) {
+      const int tt = idx / GLA_CT, c = idx % GLA_CT;
+      if (col0 + c < dv)
+        o_out[rpart * plane + ((size_t)(t0 + tt) * H + h) * dv + col0 + c] =
+            (part[tt][0][c] + part[tt][1][c]) + (part[tt][2][c] + part[tt][3][c]);
+    }
+    // The next turn's stores into sq/sk/sa/sv follow the barrier above, which every thread
+    // passes only after its last read of them; `part` is read here and written again only
+    // behind the next turn's first barrier.
+  };
+  GlaOperands<GLA_TC> even, odd;
+  if (start < end) fetch(even, start);
+  if (start + GLA_TC < end) fetch(odd, start + GLA_TC);
+  for (int t0 = start; t0 < end; t0 += 2 * GLA_TC) {
+    turn(even, t0);
+    if (t0 + GLA_TC < end) turn(odd, t0 + GLA_TC);
+  }
+#pragma unroll
+  for (int r = 0; r < 4; ++r)
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      const int i = row0 + rg * 4 + r, j = col0 + cg * 2 + c;
+      if (i < dk && j < dv) st[(size_t)i * dv + j] = S[r][c];
+    }
+}
+
+extern "C" int ta_gla_row_parts(int dk) { return (dk + GLA_RT - 1) / GLA_RT; }
+
 // proj: [nt, stride] rows holding q (H*dk) at qoff, k (H*dk) at koff, v (H*dv) at voff and the
-// low-rank decay input (rank) at aoff. a2: [H*dk, rank], a2b [H*dk]. state: [slots, H, dk, dv]
-// float32. o_out: [nt, H, dv] float32 (not yet normalised).
+// low-rank decay input (rank) at aoff. a2: [H*dk, rank], a2b [H*dk]. alpha: scratch [nt, H*dk]
+// float32. state: [slots, H, dk, dv] float32. o_out: [ta_gla_row_parts(dk), nt, H, dv] float32,
+// planes that add up to the readout (not yet normalised).
 extern "C" int ta_gla_recurrent(hipStream_t stream, int dtype, int wdtype, const void* proj, int stride,
                                 int qoff, int koff, int voff, int aoff, int rank, const void* a2,
-                                const float* a2b, float inv_tau, float qscale, float* state,
-                                const int* cu_q, const int* slots, int batch, int H, int dk, int dv,
+                                const float* a2b, float inv_tau, float qscale, float* alpha, float* state,
+                                const int* cu_q, const int* slots, int batch, int nt, int H, int dk, int dv,
                                 float* o_out) {
-  TA_REQUIRE(batch > 0 && batch <= 65535 && H > 0 && H <= 65535, "ta_gla_recurrent: bad batch %d / heads %d", batch, H);
-  TA_REQUIRE(dk >= 1 && dk <= 256 && dv >= 1 && rank >= 1, "ta_gla_recurrent: key width %d outside [1, 256]", dk);
-  const int CT = dv < 64 ? dv : 64;
-  const int Pmax = 256 / CT;
-  int need = (dk + Pmax - 1) / Pmax;
-  const int R = need <= 4 ? 4 : need <= 8 ? 8 : need <= 16 ? 16 : need <= 32 ? 32 : 64;
-  const int P = (dk + R - 1) / R;
-  const size_t lds = (size_t)GLA_TC * (3 * P * R + CT + rank + P * CT) * sizeof(float);
-  TA_REQUIRE(lds <= 64000, "ta_gla_recurrent: rank %d does not fit", rank);
-  dim3 g(batch, H, (dv + CT - 1) / CT);
-#define GLA_LAUNCH(T, TW, RR)                                                                          \
-  gla_recurrent_kernel<T, TW, RR><<<g, 256, lds, stream>>>((const T*)proj, stride, qoff, koff, voff, aoff, rank, \
-      (const TW*)a2, a2b, inv_tau, qscale, state, cu_q, slots, H, dk, dv, CT, P, o_out)
-#define GLA_BY_R(T, TW)                                     \
-  do {                                                      \
-    if (R == 4) GLA_LAUNCH(T, TW, 4);                       \
-    else if (R == 8) GLA_LAUNCH(T, TW, 8);                  \
-    else if (R == 16) GLA_LAUNCH(T, TW, 16);                \
-    else if (R == 32) GLA_LAUNCH(T, TW, 32);                \
-    else GLA_LAUNCH(T, TW, 64);                             \
-  } while (0)
-  if (dtype == TA_F32 && wdtype == TA_F32) GLA_BY_R(float, float);
-  else if (dtype == TA_BF16 && wdtype == TA_BF16) GLA_BY_R(bf16_t, bf16_t);
-  else if (dtype == TA_BF16 && wdtype == TA_F32) GLA_BY_R(bf16_t, float);
+  TA_REQUIRE(batch > 0 && batch <= 65535 && H > 0 && H <= 65535 && nt >= batch,
+             "ta_gla_recurrent: bad batch %d / heads %d / tokens %d", batch, H, nt);
+  TA_REQUIRE(dk >= 1 && dv >= 1 && rank >= 1 && rank <= 8192, "ta_gla_recurrent: bad widths %d / %d / %d", dk, dv, rank);
+  const int parts = (dk + GLA_RT - 1) / GLA_RT, tiles = (dv + GLA_CT - 1) / GLA_CT;
+  TA_REQUIRE(parts * tiles <= 65535, "ta_gla_recurrent: heads of %d x %d are too large", dk, dv);
+  const int n = H * dk;
+  dim3 gd(nt, (n + 255) / 256 < 64 ? (n + 255) / 256 : 64);
+  const size_t lds = (size_t)rank * sizeof(float);
+#define GLA_DECAY(T, TW) \
+  gla_decay_kernel<T, TW><<<gd, 256, lds, stream>>>((const T*)proj, stride, aoff, rank, (const TW*)a2, a2b, inv_tau, n, alpha)
+  if (dtype == TA_F32 && wdtype == TA_F32) GLA_DECAY(float, float);
+  else if (dtype == TA_BF16 && wdtype == TA_BF16) GLA_DECAY(bf16_t, bf16_t);
+  else if (dtype == TA_BF16 && wdtype == TA_F32) GLA_DECAY(bf16_t, float);
   else return ta_fail("ta_gla_recurrent: unsupported dtypes %d / %d", dtype, wdtype);
-#undef GLA_BY_R
-#undef GLA_LAUNCH
+#undef GLA_DECAY
+  dim3 g(batch, H, parts * tiles);
+  const size_t plane = (size_t)nt * H * dv;
+  const bool few = nt <= 8 * batch;         // at most 8 tokens a sequence on average: short chunks
+#define GLA_RUN(T, TC)                                                                                   \
+  gla_recurrent_kernel<T, TC><<<g, 256, 0, stream>>>((const T*)proj, stride, qoff, koff, voff, alpha, qscale, \
+                                                     state, cu_q, slots, H, dk, dv, tiles, plane, o_out)
+  if (dtype == TA_F32) {
+    if (few) GLA_RUN(float, 8); else GLA_RUN(float, 32);
+  } else {
+    if (few) GLA_RUN(bf16_t, 8); else GLA_RUN(bf16_t, 32);
+  }
+#undef GLA_RUN
   return ta_check_launch("ta_gla_recurrent");
 }
 
 // ------------------------------------------------------------------ gla: head norm and output gate
 template <typename T>
-__global__ __launch_bounds__(64) void gla_out_kernel(const float* __restrict__ o, const T* __restrict__ proj,
+__global__ __launch_bounds__(64) void gla_out_kernel(const float* __restrict__ o, int parts, size_t plane,
+                                                     const T* __restrict__ proj,
                                                      int stride, int goff, const float* __restrict__ w,
                                                      float eps, int H, int dv, T* __restrict__ out) {
+  extern __shared__ float row[];          // [dv]
   const size_t t = blockIdx.x;
   const int h = blockIdx.y;
   const float* src = o + (t * H + h) * dv;
   float ss = 0.f;
-  for (int c = threadIdx.x; c < dv; c += 64) ss += src[c] * src[c];
+  for (int c = threadIdx.x; c < dv; c += 64) {
+    float v = src[c];
+    for (int p = 1; p < parts; ++p) v += src[p * plane + c];
+    row[c] = v;
+    ss += v * v;
+  }
   const float f = rsqrtf(wave_sum(ss) / (float)dv + eps);
   for (int c = threadIdx.x; c < dv; c += 64) {
     const float g = to_f32(proj[t * stride + goff + h * dv + c]);
-    out[t * (size_t)(H * dv) + h * dv + c] = from_f32<T>(src[c] * f * w[c] * (g / (1.0f + expf(-g))));
+    out[t * (size_t)(H * dv) + h * dv + c] = from_f32<T>(row[c] * f * w[c] * (g / (1.0f + expf(-g))));
   }
 }
 
-// o: [nt, H, dv] float32; the gate's pre-activation sits at column goff of proj; w [dv];
-// out [nt, H*dv] = rms_norm(o per head) * w * silu(gate).
-extern "C" int ta_gla_out(hipStream_t stream, int dtype, const float* o, const void* proj, int stride,
+// o: [parts, nt, H, dv] float32 planes that add up to the readout; the gate's pre-activation sits
+// at column goff of proj; w [dv]; out [nt, H*dv] = rms_norm(o per head) * w * silu(gate).
+extern "C" int ta_gla_out(hipStream_t stream, int dtype, const float* o, int parts, const void* proj, int stride,
                           int goff, const float* w, float eps, int nt, int H, int dv, void* out) {
-  TA_REQUIRE(nt >= 0 && H > 0 && H <= 65535 && dv > 0, "ta_gla_out: bad sizes");
+  TA_REQUIRE(nt >= 0 && H > 0 && H <= 65535 && dv > 0 && dv <= 15000 && parts >= 1, "ta_gla_out: bad sizes");
   if (nt == 0) return 0;
   dim3 g(nt, H);
+  const size_t plane = (size_t)nt * H * dv, lds = (size_t)dv * sizeof(float);
   if (dtype == TA_F32)
-    gla_out_kernel<float><<<g, 64, 0, stream>>>(o, (const float*)proj, stride, goff, w, eps, H, dv, (float*)out);
+    gla_out_kernel<float><<<g, 64, lds, stream>>>(o, parts, plane, (const float*)proj, stride, goff, w, eps, H, dv, (float*)out);
   else if (dtype == TA_BF16)
-    gla_out_kernel<bf16_t><<<g, 64, 0, stream>>>(o, (const bf16_t*)proj, stride, goff, w, eps, H, dv, (bf16_t*)out);
+    gla_out_kernel<bf16_t><<<g, 64, lds, stream>>>(o, parts, plane, (const bf16_t*)proj, stride, goff, w, eps, H, dv, (bf16_t*)out);
   else
     return ta_fail("ta_gla_out: unknown dtype %d", dtype);
   return ta_check_launch("ta_gla_out");

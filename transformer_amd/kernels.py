@@ -1065,11 +1065,47 @@ def rglru_gates(yx: torch.Tensor, channels: int, x_bias, taps, conv_bias, conv_s
         c_int(batch), c_int(nt), c_int(C), c_int(nb2 // 2), _ptr(a_out), _ptr(b_out)))
 
 
+RGLRU_LIBRARY_ROWS = 256      # from this many tokens on a bfloat16 step's gates go to the matrix cores
+
+
+def rglru_gates_split(yx: torch.Tensor, channels: int, x_bias, taps, conv_bias, conv_state, gates_w,
+                      gates_b, lam, decay_scale: float, cu_q, slots, a_out, b_out, ws) -> None:
+    """``rglru_gates`` for long steps with bfloat16 weights: u is formed in float32 and split
+    into two bfloat16 numbers whose sum is u to 16 bits of mantissa; the library multiplies both
+    by the gates' blocks with float32 sums (one batched product per gate over the blocks), and
+    the two products are added before the sigmoid. ``ws``: the step's workspace."""
+    _dev(yx, "yx", contiguous=False)
+    nt, stride = _rows2d(yx, "yx")
+    C = channels
+    batch = _step_tables(cu_q, slots, nt, "rglru_gates_split")
+    _dev(gates_w, "gates_w", torch.bfloat16)
+    nb, bs, K = gates_w.shape[0] // 2, gates_w.shape[1], taps.shape[1]
+    if yx.shape[1] != 2 * C or nb * bs != C or gates_w.shape != (2 * nb, bs, bs) or nt > 65535:
+        raise KernelError(f"rglru_gates_split: shapes do not fit {C} channels / {nt} tokens")
+    u = ws.take("recurrence.u", (nt, C), torch.float32)
+    halves = ws.take("recurrence.u_split", (2, nt, C), torch.bfloat16)
+    _check(library().ta_rglru_conv_split(
+        _stream(), c_int(_code(yx.dtype)), _ptr(yx), c_int(stride), c_int(C), _ptr(x_bias), _ptr(taps),
+        _ptr(conv_bias), c_int(K), _ptr(conv_state), _ptr(cu_q), _ptr(slots), c_int(batch), c_int(nt),
+        c_int(C), _ptr(u), _ptr(halves[0]), _ptr(halves[1])))
+    g = ws.take("recurrence.gates", (2, nb, 2 * nt, bs), torch.float32)
+    lhs = halves.view(2 * nt, nb, bs).transpose(0, 1)                 # [nb, 2 nt, bs]: hi rows, then lo rows
+    for gate in range(2):
+        torch.bmm(lhs, gates_w[gate * nb:(gate + 1) * nb].transpose(1, 2), out_dtype=torch.float32, out=g[gate])
+    _check(library().ta_rglru_gates_finish(_stream(), _ptr(g), _ptr(u), _ptr(gates_b), _ptr(lam),
+                                           c_float(decay_scale), c_int(nt), c_int(C), c_int(nb),
+                                           _ptr(a_out), _ptr(b_out)))
+
+
 def rglru_scan(yx: torch.Tensor, channels: int, y_bias, x_bias, a_in, b_in, state, conv_state, cu_q,
-               slots, out: torch.Tensor) -> torch.Tensor:
+               slots, out: torch.Tensor, max_qlen: Optional[int] = None,
+               scratch: Optional[torch.Tensor] = None) -> torch.Tensor:
     """S_t = a_t S_{t-1} + b_t along every sequence; out_t = S_t * gelu_tanh(y_t + y_bias).
     ``state`` [slots, C] and ``conv_state`` [slots, K-1, C] (float32) are read and left as the
-    step's last token leaves them."""
+    step's last token leaves them. max_qlen: the most tokens a sequence brings (None: one
+    thread walks each channel whatever the length); above 64 the sequences are cut into
+    segments that are scanned side by side, which overwrites a_in and b_in and needs
+    ``scratch`` [batch, C] float32."""
     _dev(yx, "yx", contiguous=False); _dev(out, "out", yx.dtype)
     nt, stride = _rows2d(yx, "yx")
     C = channels
@@ -1081,50 +1117,66 @@ def rglru_scan(yx: torch.Tensor, channels: int, y_bias, x_bias, a_in, b_in, stat
             or state.dim() != 2 or state.shape[1] != C or conv_state.dim() != 3 or conv_state.shape[2] != C \
             or conv_state.shape[0] != state.shape[0]:
         raise KernelError(f"rglru_scan: shapes do not fit {C} channels")
+    if max_qlen is None or scratch is None:
+        max_qlen = 1
+    else:
+        _dev(scratch, "scratch", torch.float32)
+        if scratch.shape != (batch, C):
+            raise KernelError(f"rglru_scan: scratch is {tuple(scratch.shape)}, expected {(batch, C)}")
     _check(library().ta_rglru_scan(
         _stream(), c_int(_code(yx.dtype)), _ptr(yx), c_int(stride), c_int(C), _ptr(y_bias), _ptr(x_bias),
         _ptr(a_in), _ptr(b_in), _ptr(state), _ptr(conv_state), c_int(conv_state.shape[1] + 1), _ptr(cu_q),
-        _ptr(slots), c_int(batch), c_int(C), _ptr(out)))
+        _ptr(slots), c_int(batch), c_int(max_qlen), c_int(C), _ptr(scratch), _ptr(out)))
     return out
 
 
+def gla_row_parts(key_dim: int) -> int:
+    """Planes in which ``gla_recurrent`` leaves its readout (one per group of key channels that a
+    workgroup owns); ``gla_out`` adds them."""
+    return int(library().ta_gla_row_parts(c_int(key_dim)))
+
+
 def gla_recurrent(proj: torch.Tensor, heads: int, key_dim: int, value_dim: int, rank: int, a2, a2_bias,
-                  tau: float, state: torch.Tensor, cu_q, slots, o_out: torch.Tensor) -> torch.Tensor:
+                  tau: float, state: torch.Tensor, cu_q, slots, o_out: torch.Tensor,
+                  alpha: torch.Tensor) -> torch.Tensor:
     """Gated linear attention along every sequence. proj [nt, 2*H*dk + 2*H*dv + rank]: q, k, v,
     the output gate and the low-rank decay input, in that order. Per head S <- diag(alpha) S +
     k v^T with alpha = sigmoid(a2 @ low + a2_bias)^(1/tau), o = S^T (q / sqrt(dk)). ``state``
-    [slots, H, dk, dv] float32; o_out [nt, H, dv] float32."""
+    [slots, H, dk, dv] float32; ``alpha`` [nt, H*dk] float32 scratch that receives the decays;
+    o_out [gla_row_parts(dk), nt, H, dv] float32 planes that add up to the readout."""
     _dev(proj, "proj", contiguous=False)
     nt, stride = _rows2d(proj, "proj")
     H, dk, dv = heads, key_dim, value_dim
     batch = _step_tables(cu_q, slots, nt, "gla_recurrent")
     _dev(a2, "a2"); _dev(a2_bias, "a2_bias", torch.float32); _dev(state, "state", torch.float32)
-    _dev(o_out, "o_out", torch.float32)
+    _dev(o_out, "o_out", torch.float32); _dev(alpha, "alpha", torch.float32)
     if proj.shape[1] != 2 * H * dk + 2 * H * dv + rank or a2.shape != (H * dk, rank) \
             or a2_bias.shape != (H * dk,) or state.dim() != 4 or state.shape[1:] != (H, dk, dv) \
-            or o_out.shape != (nt, H, dv):
+            or o_out.shape != (gla_row_parts(dk), nt, H, dv) or alpha.shape != (nt, H * dk):
         raise KernelError(f"gla_recurrent: shapes do not fit {H} heads of {dk} / {dv}, rank {rank}: "
-                          f"proj {tuple(proj.shape)} a2 {tuple(a2.shape)} state {tuple(state.shape)}")
+                          f"proj {tuple(proj.shape)} a2 {tuple(a2.shape)} state {tuple(state.shape)} "
+                          f"o_out {tuple(o_out.shape)} alpha {tuple(alpha.shape)}")
     _check(library().ta_gla_recurrent(
         _stream(), c_int(_code(proj.dtype)), c_int(_wcode(a2, proj.dtype, "gla_recurrent")), _ptr(proj),
         c_int(stride), c_int(0), c_int(H * dk), c_int(2 * H * dk), c_int(2 * H * dk + 2 * H * dv),
-        c_int(rank), _ptr(a2), _ptr(a2_bias), c_float(1.0 / tau), c_float(float(dk) ** -0.5), _ptr(state),
-        _ptr(cu_q), _ptr(slots), c_int(batch), c_int(H), c_int(dk), c_int(dv), _ptr(o_out)))
+        c_int(rank), _ptr(a2), _ptr(a2_bias), c_float(1.0 / tau), c_float(float(dk) ** -0.5), _ptr(alpha),
+        _ptr(state), _ptr(cu_q), _ptr(slots), c_int(batch), c_int(nt), c_int(H), c_int(dk), c_int(dv),
+        _ptr(o_out)))
     return o_out
 
 
 def gla_out(o: torch.Tensor, proj: torch.Tensor, heads: int, key_dim: int, value_dim: int, weight,
             eps: float, out: torch.Tensor) -> torch.Tensor:
-    """out = rms_norm(o per head over dv) * weight * silu(gate), the gate being the fourth part
-    of the rows of ``proj`` (see ``gla_recurrent``)."""
+    """out = rms_norm(o per head over dv) * weight * silu(gate), o the sum of the planes that
+    ``gla_recurrent`` left, the gate being the fourth part of the rows of ``proj``."""
     _dev(o, "o", torch.float32); _dev(proj, "proj", contiguous=False); _dev(out, "out", proj.dtype)
     _dev(weight, "weight", torch.float32)
     nt, stride = _rows2d(proj, "proj")
     H, dk, dv = heads, key_dim, value_dim
-    if o.shape != (nt, H, dv) or out.shape != (nt, H * dv) or weight.shape != (dv,) \
+    if o.dim() != 4 or o.shape[1:] != (nt, H, dv) or out.shape != (nt, H * dv) or weight.shape != (dv,) \
             or proj.shape[1] < 2 * H * dk + 2 * H * dv:
         raise KernelError(f"gla_out: o {tuple(o.shape)} out {tuple(out.shape)} weight {tuple(weight.shape)}")
-    _check(library().ta_gla_out(_stream(), c_int(_code(proj.dtype)), _ptr(o), _ptr(proj), c_int(stride),
-                                c_int(2 * H * dk + H * dv), _ptr(weight), c_float(eps), c_int(nt), c_int(H),
-                                c_int(dv), _ptr(out)))
+    _check(library().ta_gla_out(_stream(), c_int(_code(proj.dtype)), _ptr(o), c_int(o.shape[0]), _ptr(proj),
+                                c_int(stride), c_int(2 * H * dk + H * dv), _ptr(weight), c_float(eps),
+                                c_int(nt), c_int(H), c_int(dv), _ptr(out)))
     return out

@@ -52,11 +52,17 @@ class DiagonalRecurrence(Part):
         a = ctx.ws.take("recurrence.a", (nt, C), torch.float32)
         b = ctx.ws.take("recurrence.b", (nt, C), torch.float32)
         bias = self.w["in.bias"]
-        kernels.rglru_gates(yx, C, bias[C:], self.w["conv.weight"], self.w["conv.bias"], conv_state,
-                            self.w["gates.weight"], self.w["gates.bias"], self.w["lam"],
-                            float(s.decay_scale), ctx.cu_q, ctx.slots, a, b)
+        gates = kernels.rglru_gates
+        args = ()
+        if self.dtype == torch.bfloat16 and self.w["gates.weight"].dtype == torch.bfloat16 and \
+                kernels.RGLRU_LIBRARY_ROWS <= nt <= 65535:
+            gates, args = kernels.rglru_gates_split, (ctx.ws,)      # long steps: the library's batched product
+        gates(yx, C, bias[C:], self.w["conv.weight"], self.w["conv.bias"], conv_state,
+              self.w["gates.weight"], self.w["gates.bias"], self.w["lam"],
+              float(s.decay_scale), ctx.cu_q, ctx.slots, a, b, *args)
         o = kernels.rglru_scan(yx, C, bias[:C], bias[C:], a, b, state, conv_state, ctx.cu_q, ctx.slots,
-                               ctx.ws.take("recurrence.o", (nt, C), self.dtype))
+                               ctx.ws.take("recurrence.o", (nt, C), self.dtype), ctx.max_qlen,
+                               ctx.ws.take("recurrence.s0", (ctx.batch, C), torch.float32))
         return linear_delta(o, self.w["out.weight"], ctx.ws, "recurrence.delta"), None
 
 
@@ -92,7 +98,8 @@ class GatedLinearAttention(Part):
         proj = linear(h, self.w["in.weight"], ctx.ws.take("gla.in", (nt, self.width), self.dtype))
         o = kernels.gla_recurrent(proj, H, dk, dv, s.rank, self.w["decay.weight"], self.w["decay.bias"],
                                   float(s.tau), cache.layer_state(layer), ctx.cu_q, ctx.slots,
-                                  ctx.ws.take("gla.o", (nt, H, dv), torch.float32))
+                                  ctx.ws.take("gla.o", (kernels.gla_row_parts(dk), nt, H, dv), torch.float32),
+                                  ctx.ws.take("gla.alpha", (nt, H * dk), torch.float32))
         g = kernels.gla_out(o, proj, H, dk, dv, self.w["norm.weight"], float(s.eps),
                             ctx.ws.take("gla.gated", (nt, H * dv), self.dtype))
         return linear_delta(g, self.w["out.weight"], ctx.ws, "gla.delta"), None
