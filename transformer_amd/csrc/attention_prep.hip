@@ -48,19 +48,22 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
   // Every thread reads the LDS copy and writes memory, so nothing it reads is written by another
   // thread. All loads are unconditional (a coordinate that is not rotated reads angle 0 and is
   // not changed by it), so that the loads of several turns are on their way together.
-  const float one = 1.f;
 #pragma unroll 4
   for (int i = threadIdx.x; i < nq + nk; i += 256) {
     const bool is_q = i < nq;
     const int j = is_q ? i : i - nq;
     const int head = j / dk, c = j - head * dk;
     const float f = is_q ? fq : fk;
-    const float* w = normed ? (is_q ? wq : wk) : &one;
+    const float* w = is_q ? wq : wk;
     const bool turns = ang != nullptr && c < rot;
     const int pi = turns ? (c < half ? c : c - half) : 0;
     const int shift = turns ? (c < half ? half : -half) : 0;
     const float cs = ang ? ang[2 * pi] : 1.f, sn = ang ? ang[2 * pi + 1] : 0.f;
-    const float wv = w[normed ? j : 0], wo = w[normed ? j + shift : 0];
+    float wv = 1.f, wo = 1.f;
+    if (normed) {                     // the same for every thread
+      wv = w[j];
+      wo = w[j + shift];
+    }
     float v = buf[i] * f * wv;
     const float o = buf[i + shift] * f * wo;
     if (turns) v = c < half ? v * cs - o * sn : v * cs + o * sn;

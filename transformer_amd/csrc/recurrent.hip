@@ -154,9 +154,11 @@ __global__ __launch_bounds__(256) void rglru_gates_tiled_kernel(
     // both places a tap may read (this step's rows, the sequence's memory) are asked for
     // whatever the case, at addresses that exist, and one is chosen: no load waits for a branch
     const bool on = t < nt && cc < bs;
+    // an entry that is not there computes on token 0 of the step as if it began a sequence,
+    // so that every index below stays inside its array
     const int ts = on ? t : 0, cz = on ? c : 0;
-    const int start = s_start[tt];
-    const float* cs = conv_state + ((size_t)s_slot[tt] * (K - 1)) * C;
+    const int start = on ? s_start[tt] : 0;
+    const float* cs = conv_state + ((size_t)(on ? s_slot[tt] : s_slot[0]) * (K - 1)) * C;
     const float xb = xbias[cz];
     float acc = conv_bias[cz];
     for (int j = 0; j < K; ++j) {
