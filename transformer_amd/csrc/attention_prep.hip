@@ -23,12 +23,22 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
   const int t = blockIdx.x;
   T* row = qkv + (size_t)t * stride;
   const int nq = nh * dk, nk = nkv * dk, nv = nkv * dv;
+  // Loops over a row go in groups of four turns that are known to lie inside it: a load is
+  // not asked for before the test that guards it, so turn by turn every load would wait for
+  // the one before (20 trips to memory for a row of 5,120 where 5 do).
   float sq = 0.f, sk = 0.f;
-#pragma unroll 8
-  for (int i = threadIdx.x; i < nq + nk; i += 256) {
+  auto take = [&](int i) {
     const float v = to_f32(row[i]);
     buf[i] = v;
     if (i < nq) sq += v * v; else sk += v * v;
+  };
+  {
+    int i = threadIdx.x;
+    for (; i + 768 < nq + nk; i += 1024) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) take(i + 256 * u);
+    }
+    for (; i < nq + nk; i += 256) take(i);
   }
   sq = wave_sum(sq);
   sk = wave_sum(sk);
@@ -48,8 +58,7 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
   // Every thread reads the LDS copy and writes memory, so nothing it reads is written by another
   // thread. All loads are unconditional (a coordinate that is not rotated reads angle 0 and is
   // not changed by it), so that the loads of several turns are on their way together.
-#pragma unroll 4
-  for (int i = threadIdx.x; i < nq + nk; i += 256) {
+  auto finish = [&](int i) {
     const bool is_q = i < nq;
     const int j = is_q ? i : i - nq;
     const int head = j / dk, c = j - head * dk;
@@ -72,6 +81,14 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
     } else if (dest) {
       kcache[(((size_t)page * nkv + head) * TA_PAGE + off) * dk + c] = from_f32<T>(v);
     }
+  };
+  {
+    int i = threadIdx.x;
+    for (; i + 768 < nq + nk; i += 1024) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) finish(i + 256 * u);
+    }
+    for (; i < nq + nk; i += 256) finish(i);
   }
   const float lam = lambda ? lambda[0] : 0.f;
   for (int i = threadIdx.x; i < nv; i += 256) {

@@ -147,8 +147,9 @@ __global__ __launch_bounds__(256) void rglru_gates_tiled_kernel(
     s_slot[threadIdx.x] = sl;
   }
   __syncthreads();
-#pragma unroll 4
-  for (int idx = threadIdx.x; idx < RGT_TT * bsp; idx += 256) {
+  // groups of four turns known to lie inside the tile, so that their loads are on their way
+  // together (a load is not asked for before the test that guards it)
+  auto conv = [&](int idx) {
     const int tt = idx / bsp, cc = idx - tt * bsp;
     const int t = t0 + tt, c = blk * bs + cc;
     // both places a tap may read (this step's rows, the sequence's memory) are asked for
@@ -169,6 +170,14 @@ __global__ __launch_bounds__(256) void rglru_gates_tiled_kernel(
       acc = fmaf(taps[(size_t)cz * K + j], here ? a : m, acc);
     }
     u[idx] = on ? acc : 0.f;
+  };
+  {
+    int idx = threadIdx.x;
+    for (; idx + 768 < RGT_TT * bsp; idx += 1024) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) conv(idx + 256 * q);
+    }
+    for (; idx < RGT_TT * bsp; idx += 256) conv(idx);
   }
   const int o = threadIdx.x % RGT_OC, tg = threadIdx.x / RGT_OC;      // tokens tg*4 .. tg*4+3
   const int lr = threadIdx.x / 4, lseg = (threadIdx.x % 4) * 8;       // staging: row lr, 8 inputs from lseg
