@@ -364,7 +364,8 @@ def test_layers_and_whole_prompt(name, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name,edit", [("A", None), ("B", None), ("A", "slow"), ("A", "sharp")])
+@pytest.mark.parametrize("name,edit", [("A", None), ("B", None), ("D", None), ("A", "slow"), ("A", "sharp"),
+                                       ("D", "sharp")])
 def test_cuts_agree_with_plain(name, edit, dtype):
     """Whole, portions down to two tokens, and every token alone: all against the plain model."""
     model, toks = U.engine(name, dtype, edit), U.tokens(name, 150, 2)
@@ -374,6 +375,22 @@ def test_cuts_agree_with_plain(name, edit, dtype):
         slot = cache.alloc_slot()
         got = U.run_cuts(model, cache, slot, toks, cuts)
         cache.free_slot(slot)                      # the next cut takes the same slot and pages
+        assert U.row_error(got, want).max() < U.TOL[dtype], f"cuts {cuts}"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "D"])
+def test_long_prompt_in_portions_at_the_kernels_edges(name, dtype):
+    """Portions that end at, just before and just behind the places where the recurrent kernels
+    change their ways: chunks of 8 and 32 tokens, tiles of 16, segments of 64, and the 256 tokens
+    from which a bfloat16 step forms the recurrence's gates through the library."""
+    model, toks = U.engine(name, dtype, "slow"), U.tokens(name, 400, 7)
+    want = U.plain_logits(name, dtype, "slow", tuple(toks))
+    cache = model.new_cache(512, max_slots=1)
+    for cuts in ([400], [257, 63, 65, 15], [64, 256, 33, 31, 16], [255, 129, 8, 7, 1]):
+        slot = cache.alloc_slot()
+        got = U.run_cuts(model, cache, slot, toks, cuts)
+        cache.free_slot(slot)
         assert U.row_error(got, want).max() < U.TOL[dtype], f"cuts {cuts}"
 
 

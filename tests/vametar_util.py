@@ -70,7 +70,23 @@ CFG_C = {
         _att(8, 2, 128, 64, 0.09, rot=(50000.0, 64), v_mix=True, ff=1024),
     ],
 }
-CONFIGS = {"A": (CFG_A, 11), "B": (CFG_B, 12), "C": (CFG_C, 13)}
+# a width that is no multiple of four (rows of the matrices start off 16-byte boundaries), key
+# widths the matrix-core kernels take with values as wide as the keys, narrower, and wider, and
+# a head of 160 with six query heads per kv head
+CFG_D = {
+    "architecture": "Vametar", "vocab": 77, "width": 90, "norm": {"eps": 1e-5},
+    "residual_mult": 1.3, "logit_scale": 0.5,
+    "embedding": {"bigram": {"buckets": 3, "mul_prev": 1, "mul_cur": 2}},
+    "layers": [
+        _att(4, 1, 64, 64, 0.12, rot=(10000.0, 32), ff=50),
+        _att(2, 2, 32, 16, 0.2, rot=(300.0, 32), v_mix=True),
+        _gla(2, 24, 40, 2.0, 3),
+        _att(6, 1, 160, 32, 0.08, rot=(10000.0, 160), v_mix=True, ff=33),
+        _att(2, 2, 32, 48, 0.2),
+        _rec(66, 3, 3),
+    ],
+}
+CONFIGS = {"A": (CFG_A, 11), "B": (CFG_B, 12), "C": (CFG_C, 13), "D": (CFG_D, 14)}
 STORAGE = {"float32": "F32", "bfloat16": "BF16"}
 # largest allowed rms(engine - plain) / rms(plain) over a row of logits
 TOL = {"float32": 2e-4, "bfloat16": 5e-2}

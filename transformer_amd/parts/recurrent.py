@@ -71,7 +71,7 @@ class GatedLinearAttention(Part):
 
     def __init__(self, spec, dtype, device):
         s = spec
-        if not (1 <= s.key_dim <= 256 and s.value_dim >= 1 and s.rank >= 1 and s.num_heads >= 1):
+        if not (s.key_dim >= 1 and s.value_dim >= 1 and s.rank >= 1 and s.num_heads >= 1):
             raise PartError(f"gated linear attention: heads {s.num_heads} of {s.key_dim} / {s.value_dim}, "
                             f"rank {s.rank}")
         if not s.tau > 0:
