@@ -110,6 +110,135 @@ __global__ __launch_bounds__(256) void qk_prepare_kernel(
   }
 }
 
+// The same in pieces of eight coordinates (16 bytes of bfloat16) per thread and turn, for head
+// widths that are multiples of 8 and rotations whose halves are: a row of 5,120 coordinates is
+// then two or three turns per thread instead of twenty.
+template <typename T> struct Eight;
+template <> struct Eight<float> {
+  static __device__ __forceinline__ void load(const float* p, float* v) {
+    const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+  }
+  static __device__ __forceinline__ void store(float* p, const float* v) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+    *reinterpret_cast<float4*>(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
+  }
+};
+template <> struct Eight<bf16_t> {
+  static __device__ __forceinline__ void load(const bf16_t* p, float* v) {
+    const uint4 r = *reinterpret_cast<const uint4*>(p);
+    const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      v[2 * i] = __uint_as_float(w[i] << 16);
+      v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+  }
+  static __device__ __forceinline__ void store(bf16_t* p, const float* v) {
+    uint4 r;
+    r.x = f32x2_to_bf16x2_bits(v[0], v[1]);
+    r.y = f32x2_to_bf16x2_bits(v[2], v[3]);
+    r.z = f32x2_to_bf16x2_bits(v[4], v[5]);
+    r.w = f32x2_to_bf16x2_bits(v[6], v[7]);
+    *reinterpret_cast<uint4*>(p) = r;
+  }
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void qk_prepare_vec_kernel(
+    T* __restrict__ qkv, int stride, const float* __restrict__ wq, const float* __restrict__ wk,
+    float eps, int normed, const float* __restrict__ angles, int rot,
+    const float* __restrict__ lambda, const T* __restrict__ v_first, T* __restrict__ v_keep,
+    const int* __restrict__ dest, T* __restrict__ kcache, T* __restrict__ vcache,
+    int nh, int nkv, int dk, int dv, int dvs) {
+  extern __shared__ float buf[];          // [nh*dk + nkv*dk]
+  __shared__ float red[8];
+  const int t = blockIdx.x;
+  T* row = qkv + (size_t)t * stride;
+  const int nq = nh * dk, nk = nkv * dk, nv = nkv * dv;
+  const int pieces = (nq + nk) / 8;
+  float sq = 0.f, sk = 0.f;
+  for (int p = threadIdx.x; p < pieces; p += 256) {
+    float v[8];
+    Eight<T>::load(row + 8 * p, v);
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      buf[8 * p + e] = v[e];
+      ss += v[e] * v[e];
+    }
+    if (8 * p < nq) sq += ss; else sk += ss;
+  }
+  sq = wave_sum(sq);
+  sk = wave_sum(sk);
+  if (threadIdx.x % TA_WAVE == 0) {
+    red[threadIdx.x / TA_WAVE] = sq;
+    red[4 + threadIdx.x / TA_WAVE] = sk;
+  }
+  __syncthreads();
+  float fq = 1.f, fk = 1.f;
+  if (normed) {
+    fq = rsqrtf((red[0] + red[1] + red[2] + red[3]) / (float)nq + eps);
+    fk = rsqrtf((red[4] + red[5] + red[6] + red[7]) / (float)nk + eps);
+  }
+  const int half = rot / 2;
+  const float* ang = angles ? angles + (size_t)t * half * 2 : nullptr;
+  const int page = dest ? dest[t] / TA_PAGE : 0, off = dest ? dest[t] % TA_PAGE : 0;
+  for (int p = threadIdx.x; p < pieces; p += 256) {
+    const int i = 8 * p;
+    const bool is_q = i < nq;
+    const int j = is_q ? i : i - nq;
+    const int head = j / dk, c = j - head * dk;            // the piece lies inside one head
+    const float f = is_q ? fq : fk;
+    const float* w = is_q ? wq : wk;
+    const bool turns = ang != nullptr && c < rot;          // and wholly inside or outside the rotation
+    const int shift = turns ? (c < half ? half : -half) : 0;
+    float wv[8], wo[8], cs[8], sn[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) wv[e] = wo[e] = cs[e] = 1.f, sn[e] = 0.f;
+    if (normed) {
+      Eight<float>::load(w + j, wv);
+      Eight<float>::load(w + j + shift, wo);
+    }
+    if (turns) {
+      float a[8], b[8];
+      const int pi = c < half ? c : c - half;
+      Eight<float>::load(ang + 2 * pi, a);
+      Eight<float>::load(ang + 2 * pi + 8, b);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        cs[e] = a[2 * e]; sn[e] = a[2 * e + 1];
+        cs[4 + e] = b[2 * e]; sn[4 + e] = b[2 * e + 1];
+      }
+    }
+    float out[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float v = buf[i + e] * f * wv[e], o = buf[i + shift + e] * f * wo[e];
+      out[e] = turns ? (c < half ? v * cs[e] - o * sn[e] : v * cs[e] + o * sn[e]) : v;
+    }
+    if (is_q) Eight<T>::store(row + i, out);
+    else if (dest) Eight<T>::store(kcache + (((size_t)page * nkv + head) * TA_PAGE + off) * dk + c, out);
+  }
+  const float lam = lambda ? lambda[0] : 0.f;
+  for (int i = threadIdx.x; i < nv; i += 256) {
+    float v = to_f32(row[nq + nk + i]);
+    if (v_keep) v_keep[(size_t)t * nv + i] = from_f32<T>(v);
+    if (v_first) v = (1.0f - lam) * v + lam * to_f32(v_first[(size_t)t * nv + i]);
+    if (dest) {
+      const int g = i / dv, c = i - g * dv;
+      vcache[(((size_t)page * nkv + g) * dvs + c) * TA_PAGE + off] = from_f32<T>(v);
+    }
+  }
+  if (dest && dvs > dv) {
+    const int pad = dvs - dv;
+    for (int i = threadIdx.x; i < nkv * pad; i += 256) {
+      const int g = i / pad, c = dv + (i - g * pad);
+      vcache[(((size_t)page * nkv + g) * dvs + c) * TA_PAGE + off] = from_f32<T>(0.f);
+    }
+  }
+}
+
 // qkv: [nt, stride] rows of [nh*dk | nkv*dk | nkv*dv]. wq [nh*dk], wk [nkv*dk] (used when normed).
 // angles: [nt, rot/2, 2] (cos, sin) or null. lambda: one float on the device, v_first [nt, nkv*dv]
 // (both or neither). v_keep [nt, nkv*dv] or null: receives the unmixed values. dest [nt] or null:
@@ -130,6 +259,21 @@ extern "C" int ta_qk_prepare(hipStream_t stream, int dtype, void* qkv, int strid
   TA_REQUIRE(lds <= 60000, "ta_qk_prepare: %d + %d heads of %d do not fit", nh, nkv, dk);
   if (nt == 0) return 0;
   if (rot == 0) angles = nullptr;
+  // pieces of eight: whole pieces per head and per half of the rotation, rows and tables on
+  // 16-byte boundaries (32 for float32 rows)
+  const uintptr_t all = (uintptr_t)qkv | (uintptr_t)wq | (uintptr_t)wk | (uintptr_t)angles | (uintptr_t)kcache;
+  if (dk % 8 == 0 && rot % 16 == 0 && stride % 8 == 0 && (all & 31) == 0 &&
+      (dtype == TA_F32 || dtype == TA_BF16)) {
+    if (dtype == TA_F32)
+      qk_prepare_vec_kernel<float><<<nt, 256, lds, stream>>>(
+          (float*)qkv, stride, wq, wk, eps, normed, angles, rot, lambda, (const float*)v_first, (float*)v_keep,
+          dest, (float*)kcache, (float*)vcache, nh, nkv, dk, dv, dvs);
+    else
+      qk_prepare_vec_kernel<bf16_t><<<nt, 256, lds, stream>>>(
+          (bf16_t*)qkv, stride, wq, wk, eps, normed, angles, rot, lambda, (const bf16_t*)v_first, (bf16_t*)v_keep,
+          dest, (bf16_t*)kcache, (bf16_t*)vcache, nh, nkv, dk, dv, dvs);
+    return ta_check_launch("ta_qk_prepare");
+  }
   if (dtype == TA_F32)
     qk_prepare_kernel<float><<<nt, 256, lds, stream>>>(
         (float*)qkv, stride, wq, wk, eps, normed, angles, rot, lambda, (const float*)v_first, (float*)v_keep,
