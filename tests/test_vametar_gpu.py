@@ -115,6 +115,31 @@ def test_gated_add_and_norm(dtype):
     np.testing.assert_allclose(out.float().cpu().numpy(), P.unit_rms(v, eps) * w, atol=_atol(dtype))
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_token_shift_on_the_norm_of_single_token_steps(dtype):
+    """The norm's kernel takes the shift over when every sequence brings one token: the same
+    rows and the same state as the norm followed by the shift's own kernel."""
+    from transformer_amd import kernels as K
+    td = torch.float32 if dtype == "float32" else torch.bfloat16
+    rng = np.random.default_rng(9)
+    nt, d, eps = 5, 72, 1e-5
+    x, delta, gate = (rng.standard_normal((nt, d)) for _ in range(3))
+    w, mu = 1 + 0.1 * rng.standard_normal(d), rng.uniform(0, 1, d)
+    st = rng.standard_normal((7, d))
+    slots, cu = _t([6, 0, 3, 2, 5], torch.int32), _tables([1] * nt)
+    pend = lambda: K.GatedDelta(_t(delta), None, _t(gate), None, 0.7)
+    xa, ha, sa = _t(x), torch.empty(nt, d, dtype=td, device=DEV), _t(st)
+    K.gated_add_rmsnorm(xa, _t(w), eps, ha, pend())
+    hsa = K.token_shift(ha, torch.empty_like(ha), _t(mu), sa, cu, slots)
+    xb, hb, sb, hsb = _t(x), torch.empty(nt, d, dtype=td, device=DEV), _t(st), torch.empty(nt, d, dtype=td, device=DEV)
+    K.gated_add_rmsnorm(xb, _t(w), eps, hb, pend(), shift=(_t(mu), sb, slots, hsb))
+    for a, b in ((xa, xb), (ha, hb), (hsa, hsb), (sa, sb)):
+        assert torch.equal(a, b)
+    v = x + 0.7 * P.sigmoid(gate) * delta
+    h = P.unit_rms(v, eps) * w
+    np.testing.assert_allclose(hsb.float().cpu().numpy(), h + (st[[6, 0, 3, 2, 5]] - h) * mu, atol=_atol(dtype))
+
+
 def _paged(model_dtype, pages, nkv, dk, dv):
     from transformer_amd.kernels import PAGE
     kc = torch.zeros(pages, nkv, PAGE, dk, dtype=model_dtype, device=DEV)

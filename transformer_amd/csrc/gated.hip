@@ -74,7 +74,9 @@ __global__ __launch_bounds__(1024) void gated_add_rmsnorm_wide_kernel(
     float* __restrict__ x, const float* __restrict__ delta, int planes, size_t plane,
     const float* __restrict__ delta_bias, const float* __restrict__ gate,
     const float* __restrict__ gate_bias, float mult, const float* __restrict__ weight,
-    const int* __restrict__ rows, TO* __restrict__ out, int d, float eps, int store) {
+    const int* __restrict__ rows, TO* __restrict__ out, int d, float eps, int store,
+    const float* __restrict__ mu, float* __restrict__ state, const int* __restrict__ slots,
+    TO* __restrict__ shifted) {
   __shared__ float red[16];
   const int i = blockIdx.x;
   const size_t r = rows ? (size_t)rows[i] : (size_t)i;
@@ -113,32 +115,52 @@ __global__ __launch_bounds__(1024) void gated_add_rmsnorm_wide_kernel(
   const float f = rsqrtf(tot / (float)d + eps);
   if (on) {
     TO* o = out + (size_t)i * d + c;
-    o[0] = from_f32<TO>(v.x * f * w.x);
-    o[1] = from_f32<TO>(v.y * f * w.y);
-    o[2] = from_f32<TO>(v.z * f * w.z);
-    o[3] = from_f32<TO>(v.w * f * w.w);
+    const TO h[4] = {from_f32<TO>(v.x * f * w.x), from_f32<TO>(v.y * f * w.y), from_f32<TO>(v.z * f * w.z),
+                     from_f32<TO>(v.w * f * w.w)};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = h[e];
+    if (shifted) {
+      // steps of single tokens: row i is sequence i's only token, so the row before it is the
+      // sequence's state row, which then takes this row (the token shift, without a kernel of
+      // its own)
+      float* st = state + (size_t)slots[i] * d + c;
+      const float4 prev = *reinterpret_cast<const float4*>(st);
+      const float4 m = *reinterpret_cast<const float4*>(mu + c);
+      const float cur[4] = {to_f32(h[0]), to_f32(h[1]), to_f32(h[2]), to_f32(h[3])};
+      const float pv[4] = {prev.x, prev.y, prev.z, prev.w}, mv[4] = {m.x, m.y, m.z, m.w};
+      TO* hs = shifted + (size_t)i * d + c;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) hs[e] = from_f32<TO>(cur[e] + (pv[e] - cur[e]) * mv[e]);
+      *reinterpret_cast<float4*>(st) = make_float4(cur[0], cur[1], cur[2], cur[3]);
+    }
   }
 }
 
-extern "C" int ta_gated_add_rmsnorm(hipStream_t stream, int out_dtype, float* x, const float* delta,
+static int gated_add_rmsnorm_launch(hipStream_t stream, int out_dtype, float* x, const float* delta,
                                     int planes, long long plane, const float* delta_bias,
                                     const float* gate, const float* gate_bias, float mult,
                                     const float* weight, const int* rows, void* out, int n_out, int d,
-                                    float eps, int store) {
+                                    float eps, int store, const float* mu, float* state, const int* slots,
+                                    void* shifted) {
   TA_REQUIRE(n_out >= 0 && d > 0 && d <= 16000, "ta_gated_add_rmsnorm: bad sizes n=%d d=%d", n_out, d);
   TA_REQUIRE(planes >= 1 && planes <= TA_MAX_PLANES, "ta_gated_add_rmsnorm: %d planes", planes);
   if (n_out == 0) return 0;
   const bool aligned = (((uintptr_t)x | (uintptr_t)delta | (uintptr_t)gate | (uintptr_t)gate_bias |
-                         (uintptr_t)delta_bias | (uintptr_t)weight | (uintptr_t)((size_t)plane * 4)) & 15) == 0;
+                         (uintptr_t)delta_bias | (uintptr_t)weight | (uintptr_t)((size_t)plane * 4) |
+                         (uintptr_t)mu | (uintptr_t)state) & 15) == 0;
   if (d % 4 == 0 && d <= 4096 && aligned && (out_dtype == TA_F32 || out_dtype == TA_BF16)) {
     if (out_dtype == TA_F32)
       gated_add_rmsnorm_wide_kernel<float><<<n_out, 1024, 0, stream>>>(
-          x, delta, planes, (size_t)plane, delta_bias, gate, gate_bias, mult, weight, rows, (float*)out, d, eps, store);
+          x, delta, planes, (size_t)plane, delta_bias, gate, gate_bias, mult, weight, rows, (float*)out, d, eps, store,
+          mu, state, slots, (float*)shifted);
     else
       gated_add_rmsnorm_wide_kernel<bf16_t><<<n_out, 1024, 0, stream>>>(
-          x, delta, planes, (size_t)plane, delta_bias, gate, gate_bias, mult, weight, rows, (bf16_t*)out, d, eps, store);
+          x, delta, planes, (size_t)plane, delta_bias, gate, gate_bias, mult, weight, rows, (bf16_t*)out, d, eps, store,
+          mu, state, slots, (bf16_t*)shifted);
     return ta_check_launch("ta_gated_add_rmsnorm");
   }
+  TA_REQUIRE(shifted == nullptr, "ta_gated_add_rmsnorm_shift: rows of %d coordinates are not taken (a multiple "
+             "of 4 up to 4096, on 16-byte boundaries)", d);
   const size_t lds = (size_t)d * sizeof(float);
   if (out_dtype == TA_F32)
     gated_add_rmsnorm_kernel<float><<<n_out, 256, lds, stream>>>(
@@ -149,6 +171,28 @@ extern "C" int ta_gated_add_rmsnorm(hipStream_t stream, int out_dtype, float* x,
   else
     return ta_fail("ta_gated_add_rmsnorm: unknown dtype %d", out_dtype);
   return ta_check_launch("ta_gated_add_rmsnorm");
+}
+
+extern "C" int ta_gated_add_rmsnorm(hipStream_t stream, int out_dtype, float* x, const float* delta,
+                                    int planes, long long plane, const float* delta_bias,
+                                    const float* gate, const float* gate_bias, float mult,
+                                    const float* weight, const int* rows, void* out, int n_out, int d,
+                                    float eps, int store) {
+  return gated_add_rmsnorm_launch(stream, out_dtype, x, delta, planes, plane, delta_bias, gate, gate_bias, mult,
+                                  weight, rows, out, n_out, d, eps, store, nullptr, nullptr, nullptr, nullptr);
+}
+
+// The same for a step in which every sequence brings ONE token (row i belongs to slots[i]),
+// with the token shift behind the norm: shifted[i] = out[i] + (state[slots[i]] - out[i]) * mu,
+// then state[slots[i]] = out[i]. Rows of a multiple of 4 up to 4,096 coordinates only.
+extern "C" int ta_gated_add_rmsnorm_shift(hipStream_t stream, int out_dtype, float* x, const float* delta,
+                                          int planes, long long plane, const float* delta_bias,
+                                          const float* gate, const float* gate_bias, float mult,
+                                          const float* weight, void* out, int n_out, int d, float eps,
+                                          const float* mu, float* state, const int* slots, void* shifted) {
+  TA_REQUIRE(mu && state && slots && shifted, "ta_gated_add_rmsnorm_shift: shift operands missing");
+  return gated_add_rmsnorm_launch(stream, out_dtype, x, delta, planes, plane, delta_bias, gate, gate_bias, mult,
+                                  weight, nullptr, out, n_out, d, eps, 1, mu, state, slots, shifted);
 }
 
 // ------------------------------------------------------------------ token shift

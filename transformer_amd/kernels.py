@@ -853,12 +853,22 @@ class GatedDelta:
         return x + self.mult * d
 
 
+def norm_shift_fuses(d: int) -> bool:
+    """Whether ``gated_add_rmsnorm`` takes the token shift of a single-token step over."""
+    return d % 4 == 0 and d <= 4096
+
+
 def gated_add_rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor,
                       pending: Optional[GatedDelta] = None,
-                      rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+                      rows: Optional[torch.Tensor] = None, shift=None) -> torch.Tensor:
     """v = x[r] + pending (see ``GatedDelta``); out[i] = v / sqrt(mean(v^2) + eps) * weight.
     Without ``rows`` v is stored back into x; with ``rows`` (int32) only those rows are
-    normalised and x is left as it is."""
+    normalised and x is left as it is.
+
+    shift = (mu [d], state [slots, d] float32, slots int32 [nt], shifted [nt, d]): for a step
+    in which every sequence brings one token (row i belongs to slots[i]) the token shift runs
+    behind the norm in the same kernel: shifted[i] = out[i] + (state[slots[i]] - out[i]) * mu,
+    and the state row takes out[i]. Only where ``norm_shift_fuses(d)``."""
     _dev(x, "x", torch.float32); _dev(weight, "weight", torch.float32); _dev(out, "out")
     nt, d = x.shape
     if weight.shape != (d,):
@@ -888,6 +898,19 @@ def gated_add_rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: to
             _dev(gate, "gate", torch.float32)
             if gate.shape != x.shape:
                 raise KernelError(f"gated_add_rmsnorm: gate is {tuple(gate.shape)}, x {tuple(x.shape)}")
+    if shift is not None:
+        mu, state, slots, shifted = shift
+        _dev(mu, "mu", torch.float32); _dev(state, "state", torch.float32)
+        _dev(slots, "slots", torch.int32); _dev(shifted, "shifted", out.dtype)
+        if rows is not None or not norm_shift_fuses(d) or mu.shape != (d,) or state.dim() != 2 \
+                or state.shape[1] != d or slots.numel() != nt or shifted.shape != (nt, d):
+            raise KernelError(f"gated_add_rmsnorm: the token shift cannot be taken over for rows of {d} "
+                              f"(mu {tuple(mu.shape)}, state {tuple(state.shape)}, {slots.numel()} slots)")
+        _check(library().ta_gated_add_rmsnorm_shift(
+            _stream(), c_int(_code(out.dtype)), _ptr(x), _ptr(delta), c_int(planes), c_longlong(plane),
+            _ptr(dbias), _ptr(gate), _ptr(gbias), c_float(mult), _ptr(weight), _ptr(out), c_int(n_out),
+            c_int(d), c_float(eps), _ptr(mu), _ptr(state), _ptr(slots), _ptr(shifted)))
+        return out
     _check(library().ta_gated_add_rmsnorm(
         _stream(), c_int(_code(out.dtype)), _ptr(x), _ptr(delta), c_int(planes), c_longlong(plane),
         _ptr(dbias), _ptr(gate), _ptr(gbias), c_float(mult), _ptr(weight), _ptr(rows), _ptr(out),

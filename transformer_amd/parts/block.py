@@ -169,15 +169,25 @@ class GatedPreNormBlock(Part):
     def run(self, x, pending, ctx, cache, layer, writes_cache=True, after=None):
         s = self.spec
         h = ctx.ws.take("block.h", x.shape, self.dtype)
-        with span(ctx, "norm"):
-            self.norm1.run(x, h, pending[0], pending[1])
         layers = list(layer) if isinstance(layer, (list, tuple)) else ([] if layer is None else [layer])
+        hs = h
+        shift_state = cache.layer_state(layers.pop(0)) if s.token_shift else None
+        # a step of single tokens: the shift rides on the norm's kernel (the row before a
+        # sequence's only token is its state row)
+        on_norm = s.token_shift and ctx.all_single and kernels.norm_shift_fuses(self.hidden) \
+            and isinstance(pending, tuple) and getattr(self.norm1, "takes_shift", False)
+        with span(ctx, "norm"):
+            if on_norm:
+                hs = ctx.ws.take("block.hs", x.shape, self.dtype)
+                self.norm1.run(x, h, pending[0], pending[1],
+                               shift=(self.w["shift"], shift_state, ctx.slots, hs))
+            else:
+                self.norm1.run(x, h, pending[0], pending[1])
         with span(ctx, "gate"):
             gate, gbias = self._gate(h, "gate1", ctx)
-            hs = h
-            if s.token_shift:
+            if s.token_shift and not on_norm:
                 hs = kernels.token_shift(h, ctx.ws.take("block.hs", x.shape, self.dtype), self.w["shift"],
-                                         cache.layer_state(layers.pop(0)), ctx.cu_q, ctx.slots)
+                                         shift_state, ctx.cu_q, ctx.slots)
         need = self.mixer.cache_need()
         mixer_layer = None if need is None else tuple(layers) if isinstance(need, (list, tuple)) \
             else layers[0]

@@ -19,6 +19,7 @@ from .base import Part, register_part
 
 class RMSNorm(Part):
     graph_safe = True
+    takes_shift = True      # ``run(..., shift=)``: a single-token step's token shift in the norm's kernel
 
     def __init__(self, spec, dtype, device):
         self.size, self.eps, self.dtype = spec.size, float(spec.eps), dtype
@@ -27,10 +28,15 @@ class RMSNorm(Part):
         return {"weight": Param((self.size,), "vector", init="around_one")}
 
     def run(self, x: torch.Tensor, out: torch.Tensor, delta: Optional[torch.Tensor] = None,
-            delta_bias: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None):
+            delta_bias: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None, shift=None):
         """x: float32 [nt, size], updated in place by the pending delta unless
         ``rows`` selects the rows to normalise. out: engine dtype. ``delta`` may be a
         ``kernels.GatedDelta`` (what a gated sublayer leaves to be added)."""
+        if shift is not None:
+            # a single-token step's token shift rides on the norm (``kernels.gated_add_rmsnorm``)
+            if delta is not None and not isinstance(delta, kernels.GatedDelta):
+                delta = kernels.GatedDelta(delta, delta_bias)
+            return kernels.gated_add_rmsnorm(x, self.gain(), self.eps, out, delta, rows, shift)
         if isinstance(delta, kernels.GatedDelta):
             return kernels.gated_add_rmsnorm(x, self.gain(), self.eps, out, delta, rows)
         return kernels.add_rmsnorm(x, self.gain(), self.eps, out, delta, delta_bias, rows)
