@@ -148,3 +148,20 @@ def test_plain_model_is_causal():
     toks = U.tokens("B", 12, 0)
     a, b = m.forward(toks), m.forward(toks[:7])
     np.testing.assert_allclose(a[:7], b, atol=1e-10)
+
+
+def test_bench_shapes_of_the_design_option_are_valid_models():
+    """``bench.py --design vametar`` builds these: every layer kind alone and the Llama layer of
+    the same width, heads and feed-forward."""
+    import bench
+    import transformer_amd as ta
+    for size, (base, kinds, llama) in bench.vametar_shapes().items():
+        for kind, layer in kinds.items():
+            cfg = ta.VametarConfig.from_dict({**base, "layers": [layer] * 2})
+            spec = cfg.model_spec()
+            assert len(spec.blocks) == 2 and spec.hidden == base["width"], (size, kind)
+        lc = ta.LlamaConfig.from_dict({**llama, "num_hidden_layers": 2})
+        att = kinds["attention"]["mixer"]
+        assert (lc.hidden, lc.num_heads, lc.num_kv_heads, lc.head_dim) == \
+            (base["width"], att["heads"], att["kv_heads"], att["dim"])
+        assert lc.intermediate == kinds["attention"]["mlp"]["ff"]
