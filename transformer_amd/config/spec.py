@@ -235,3 +235,135 @@ class GatedBlockSpec:
     gated: bool = True
     token_shift: bool = True
     kind: str = "gated_prenorm"
+
+
+# ---------------------------------------------------------------------------------------------
+# Parts that the Kunitar decoder added; as above, every size and constant is a field.
+
+@dataclass(frozen=True)
+class EmbedScaleSpec:
+    """An ``after_embed`` part: the embedded rows are multiplied by ``scale``."""
+    scale: float
+    kind: str = "embed_scale"
+
+
+@dataclass(frozen=True)
+class TokenSideTableSpec:
+    """An ``after_embed`` part: a second table [vocab, width] indexed by the step's tokens,
+    whose gathered rows (float32) the blocks' ``TokenSideSpec`` parts read for the rest of
+    the step, each its own range of columns."""
+    vocab: int
+    width: int
+    kind: str = "token_side_table"
+
+
+@dataclass(frozen=True)
+class ChainSpec:
+    """Several ``after_embed`` / ``on_logits`` parts run one after another; part i's
+    parameters are named ``<i>.<name>``."""
+    parts: Tuple[object, ...]
+    kind: str = "chain"
+
+
+@dataclass(frozen=True)
+class TokenSideSpec:
+    """x += rms_norm(P (gelu_tanh(G x) * e)) * w: e = columns [offset, offset + dim) of the
+    step's side-table rows, G [dim, hidden] reads the residual stream itself, P [hidden, dim]."""
+    hidden: int
+    dim: int
+    offset: int
+    eps: float
+    kind: str = "token_side"
+
+
+@dataclass(frozen=True)
+class MLPSpec:
+    """down(act(up(h))); activation "gelu" (erf), "gelu_tanh", "relu2" (relu squared), "silu"."""
+    hidden: int
+    intermediate: int
+    activation: str = "gelu"
+    kind: str = "mlp"
+
+
+@dataclass(frozen=True)
+class RoutedMLPSpec:
+    """``experts`` feed-forward layers down(act(up(.))) of width ``intermediate``, of which a
+    token uses the ``top`` with the largest router scores. score "sigmoid" (each expert's own)
+    or "softmax" (over the experts); renormalize: the chosen scores are divided by their sum;
+    weight_on "input": an expert is applied to weight * h, "output": its result is weighted.
+    shared_intermediate: a further expert of that width that every token uses (None: none);
+    shared_gate: its result is multiplied by sigmoid(g . h), one number per token."""
+    hidden: int
+    experts: int
+    top: int
+    intermediate: int
+    activation: str = "relu2"
+    score: str = "sigmoid"
+    renormalize: bool = False
+    weight_on: str = "input"
+    shared_intermediate: Optional[int] = None
+    shared_gate: bool = True
+    kind: str = "routed_mlp"
+
+
+@dataclass(frozen=True)
+class LatentAttentionSpec:
+    """Softmax attention whose keys and values are linear maps of ONE cached latent per token.
+
+    Queries: cq = rms_norm(Dq h) (q_rank wide), q = Uq cq, per head [nope_dim unrotated |
+    rope_dim rotated]. Keys/values: Dkv h = [kv_rank | rope_dim]; the first part, RMS-normed,
+    is the latent c, the second, rotated, is a key part that all heads share; per head k =
+    [Uk c | shared part], v = Uv c (value_dim). Rotation: the first rot_dims coordinates of a
+    rotated part in pairs (2i, 2i + 1) by position * rot_base^(-2i/rot_dims). window: a query
+    at p reads keys in (p - window, p]; None: all. gated: head h's result is multiplied by
+    sigmoid(g_h . h). own_kv False: no Dkv; the layer reads the rows that the layer whose cache
+    it borrows stored (its schedule entry names it). cache_window: the window the cache layer
+    is kept for (the widest of the layers that read it; None: everything)."""
+    hidden: int
+    num_heads: int
+    nope_dim: int
+    rope_dim: int
+    value_dim: int
+    q_rank: int
+    kv_rank: int
+    scale: float
+    eps: float
+    rot_dims: int
+    rot_base: float = 10000.0
+    window: Optional[int] = None
+    cache_window: Optional[int] = None
+    gated: bool = True
+    own_kv: bool = True
+    kind: str = "latent_attention"
+
+
+@dataclass(frozen=True)
+class BonusRecurrenceSpec:
+    """Per head a matrix state S [head_dim, head_dim]: o_t = (S + diag(u) k_t v_t^T)^T r_t, then
+    S <- diag(w_t) S + k_t v_t^T, w_t = exp(-exp(W2 tanh(W1 m_w) + w0)) (W1 maps to decay_rank
+    numbers). r, k, v, the output gate and the decay each read a token-shifted row of their
+    own, h_t + (h_{t-1} - h_t) * mu_s. o is divided by its root mean square per head, times a
+    weight per channel, times silu(gate), then projected."""
+    hidden: int
+    num_heads: int
+    head_dim: int
+    decay_rank: int
+    eps: float
+    kind: str = "bonus_recurrence"
+
+
+@dataclass(frozen=True)
+class SandwichBlockSpec:
+    """x += scale1 * norm1b(mixer(norm1(x))); x += scale2 * norm2b(ffn(norm2(x))); then the
+    optional ``side`` part adds what it derives from the stream and the step's tokens.
+    layer_scale: scale1 / scale2 are learned vectors (else 1). ffn None: one sublayer."""
+    norm1: object
+    mixer: object
+    norm1b: object
+    norm2: object = None
+    ffn: object = None
+    norm2b: object = None
+    side: object = None
+    hidden: int = 0
+    layer_scale: bool = True
+    kind: str = "sandwich"

@@ -198,9 +198,9 @@ extern "C" int ta_gated_add_rmsnorm_shift(hipStream_t stream, int out_dtype, flo
 // ------------------------------------------------------------------ token shift
 template <typename T>
 __global__ __launch_bounds__(256) void token_shift_kernel(
-    const T* __restrict__ h, T* __restrict__ hs, const float* __restrict__ mu,
+    const T* __restrict__ h, T* __restrict__ hs, const float* __restrict__ mu, int n_mu,
     float* __restrict__ state, const int* __restrict__ cu_q, const int* __restrict__ slots,
-    int batch, int d) {
+    int batch, int nt, int d) {
   const int t = blockIdx.x;
   const int b = seq_of_token(cu_q, batch, t);
   const int first = cu_q[b], last = cu_q[b + 1] - 1;
@@ -214,23 +214,33 @@ __global__ __launch_bounds__(256) void token_shift_kernel(
     } else {
       prev = to_f32(h[(size_t)(t - 1) * d + c]);
     }
-    hs[(size_t)t * d + c] = from_f32<T>(cur + (prev - cur) * mu[c]);
+    for (int s = 0; s < n_mu; ++s)
+      hs[((size_t)s * nt + t) * d + c] = from_f32<T>(cur + (prev - cur) * mu[(size_t)s * d + c]);
   }
 }
 
-// h, hs: [nt, d]; mu: [d]; state: [slots, d] float32, the sequence's last unshifted row.
-extern "C" int ta_token_shift(hipStream_t stream, int dtype, const void* h, void* hs, const float* mu,
-                              float* state, const int* cu_q, const int* slots, int batch, int nt, int d) {
-  TA_REQUIRE(batch > 0 && nt >= batch && d > 0, "ta_token_shift: bad sizes batch=%d nt=%d d=%d", batch, nt, d);
+// h: [nt, d]; mu: [n_mu, d]; hs: [n_mu, nt, d], one shifted copy of the rows per mu; state:
+// [slots, d] float32, the sequence's last unshifted row.
+extern "C" int ta_token_shift_multi(hipStream_t stream, int dtype, const void* h, void* hs, const float* mu,
+                                    int n_mu, float* state, const int* cu_q, const int* slots, int batch,
+                                    int nt, int d) {
+  TA_REQUIRE(batch > 0 && nt >= batch && d > 0 && n_mu >= 1 && n_mu <= 64,
+             "ta_token_shift: bad sizes batch=%d nt=%d d=%d mus=%d", batch, nt, d, n_mu);
   // few rows: a column tile per workgroup, so that a thread makes one trip to memory
   dim3 g(nt, nt <= 256 ? (d + 255) / 256 : 1);
   if (dtype == TA_F32)
-    token_shift_kernel<float><<<g, 256, 0, stream>>>((const float*)h, (float*)hs, mu, state, cu_q, slots, batch, d);
+    token_shift_kernel<float><<<g, 256, 0, stream>>>((const float*)h, (float*)hs, mu, n_mu, state, cu_q, slots, batch, nt, d);
   else if (dtype == TA_BF16)
-    token_shift_kernel<bf16_t><<<g, 256, 0, stream>>>((const bf16_t*)h, (bf16_t*)hs, mu, state, cu_q, slots, batch, d);
+    token_shift_kernel<bf16_t><<<g, 256, 0, stream>>>((const bf16_t*)h, (bf16_t*)hs, mu, n_mu, state, cu_q, slots, batch, nt, d);
   else
     return ta_fail("ta_token_shift: unknown dtype %d", dtype);
   return ta_check_launch("ta_token_shift");
+}
+
+// The same with one mu: hs [nt, d].
+extern "C" int ta_token_shift(hipStream_t stream, int dtype, const void* h, void* hs, const float* mu,
+                              float* state, const int* cu_q, const int* slots, int batch, int nt, int d) {
+  return ta_token_shift_multi(stream, dtype, h, hs, mu, 1, state, cu_q, slots, batch, nt, d);
 }
 
 // ------------------------------------------------------------------ hashed pair embedding

@@ -16,7 +16,11 @@ __global__ __launch_bounds__(256) void gemm_simple_kernel(const T* __restrict__ 
                                                           const TW* __restrict__ W, int ldw,
                                                           const float* __restrict__ bias,
                                                           TC* __restrict__ C, int ldc, int M,
-                                                          int N, int K) {
+                                                          int N, int K, long long sa, long long sw,
+                                                          long long sc) {
+  A += (size_t)blockIdx.z * sa;
+  W += (size_t)blockIdx.z * sw;
+  C += (size_t)blockIdx.z * sc;
   __shared__ float As[BK][BM + 4];
   __shared__ float Ws[BK][BN + 4];
   const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
@@ -68,18 +72,21 @@ __global__ __launch_bounds__(256) void gemm_simple_kernel(const T* __restrict__ 
 }
 
 // in_dtype: type of A; w_dtype: type of W (a bfloat16 engine keeps a matrix that its file
-// stores in 32 bits as it is: bfloat16 A with float32 W); out_dtype: type of C.
-extern "C" int ta_gemm_simple(hipStream_t stream, int in_dtype, int w_dtype, int out_dtype,
-                              const void* A, int lda, const void* W, int ldw, const float* bias,
-                              void* C, int ldc, int M, int N, int K) {
-  TA_REQUIRE(M >= 0 && N > 0 && K > 0, "ta_gemm_simple: bad sizes M=%d N=%d K=%d", M, N, K);
+// stores in 32 bits as it is: bfloat16 A with float32 W); out_dtype: type of C. ``batch``
+// products side by side: product i reads A + i*sa, W + i*sw and writes C + i*sc (elements).
+extern "C" int ta_gemm_simple_batched(hipStream_t stream, int in_dtype, int w_dtype, int out_dtype,
+                                      const void* A, int lda, long long sa, const void* W, int ldw,
+                                      long long sw, const float* bias, void* C, int ldc, long long sc,
+                                      int M, int N, int K, int batch) {
+  TA_REQUIRE(M >= 0 && N > 0 && K > 0 && batch >= 1 && batch <= 65535,
+             "ta_gemm_simple: bad sizes M=%d N=%d K=%d batch=%d", M, N, K, batch);
   TA_REQUIRE(lda >= K && ldw >= K && ldc >= N, "ta_gemm_simple: leading dimensions too small");
   if (M == 0) return 0;
-  dim3 g((N + BN - 1) / BN, (M + BM - 1) / BM), b(256);
+  dim3 g((N + BN - 1) / BN, (M + BM - 1) / BM, batch), b(256);
   TA_REQUIRE(g.y <= 65535, "ta_gemm_simple: M=%d too large for one launch", M);
 #define LAUNCH(T, TW, TC)                                                                        \
   gemm_simple_kernel<T, TW, TC><<<g, b, 0, stream>>>((const T*)A, lda, (const TW*)W, ldw, bias,   \
-                                                     (TC*)C, ldc, M, N, K)
+                                                     (TC*)C, ldc, M, N, K, sa, sw, sc)
   if (in_dtype == TA_F32 && w_dtype == TA_F32 && out_dtype == TA_F32) LAUNCH(float, float, float);
   else if (in_dtype == TA_BF16 && w_dtype == TA_BF16 && out_dtype == TA_BF16) LAUNCH(bf16_t, bf16_t, bf16_t);
   else if (in_dtype == TA_BF16 && w_dtype == TA_BF16 && out_dtype == TA_F32) LAUNCH(bf16_t, bf16_t, float);
@@ -88,4 +95,11 @@ extern "C" int ta_gemm_simple(hipStream_t stream, int in_dtype, int w_dtype, int
   else return ta_fail("ta_gemm_simple: unsupported dtypes a=%d w=%d out=%d", in_dtype, w_dtype, out_dtype);
 #undef LAUNCH
   return ta_check_launch("ta_gemm_simple");
+}
+
+extern "C" int ta_gemm_simple(hipStream_t stream, int in_dtype, int w_dtype, int out_dtype,
+                              const void* A, int lda, const void* W, int ldw, const float* bias,
+                              void* C, int ldc, int M, int N, int K) {
+  return ta_gemm_simple_batched(stream, in_dtype, w_dtype, out_dtype, A, lda, 0, W, ldw, 0, bias, C, ldc, 0,
+                                M, N, K, 1);
 }

@@ -1,0 +1,319 @@
+// Attention over a cache that keeps ONE row per token for all heads: a latent c [rank] from
+// which every head's unrotated key and value are linear maps (k_h = Uk_h c, v_h = Uv_h c), and
+// a rotated key part [rot] that the heads share. The maps are applied to the query and to the
+// result instead of to the cached rows:
+//
+//   score(h, i, j) = ((Uk_h^T q_h,i) . c_j + qrot_h,i . krot_j) * scale
+//   out_h,i        = Uv_h (sum_j p(h, i, j) c_j)
+//
+// so the kernels here see one "key" row [rank + rot] per token, queries of the same width,
+// and return the weighted sums of the first `rank` coordinates.
+//
+//   latent_prepare   : from the rows of a step's first product: RMS norm of the query latent;
+//                      RMS norm of the key/value latent and rotation of the shared key part,
+//                      both stored into the cache row of the token
+//   latent_query_rot : the rotated part of every head's query, rotated, into the last `rot`
+//                      coordinates of the wide query rows
+//   latent_attention : causal (windowed) softmax attention of the wide queries over the
+//                      cached rows, float32 on the vector ALU, an output gate per (token, head)
+//
+// Rotation: coordinates (2i, 2i + 1), i < dims / 2, of a rotated part turn by the token's
+// angle i; angles come as (cos, sin) float32 [nt, dims / 2, 2]. Everything between loads and
+// the one rounding of each result is float32. Keys are walked in chunks of 32 aligned to
+// absolute positions, so a row's bits depend on its own query and keys only.
+#include "common.h"
+
+__device__ __forceinline__ float la_block_sum(float v, float* red) {
+  v = wave_sum(v);
+  const int w = threadIdx.x / TA_WAVE;
+  __syncthreads();
+  if (threadIdx.x % TA_WAVE == 0) red[w] = v;
+  __syncthreads();
+  float s = 0.f;
+  for (int i = 0; i < (int)(blockDim.x / TA_WAVE); ++i) s += red[i];
+  return s;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void latent_prepare_kernel(
+    const T* __restrict__ proj, int stride, int q_rank, const float* __restrict__ qw, T* __restrict__ cq,
+    int kvoff, int rank, int rot, int rot_dims, const float* __restrict__ kw, float eps,
+    const float* __restrict__ angles, const int* __restrict__ dest, T* __restrict__ kcache) {
+  __shared__ float red[4];
+  const size_t t = blockIdx.x;
+  const T* row = proj + t * stride;
+  if (q_rank > 0) {
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < q_rank; c += 256) {
+      const float v = to_f32(row[c]);
+      ss += v * v;
+    }
+    const float f = rsqrtf(la_block_sum(ss, red) / (float)q_rank + eps);
+    for (int c = threadIdx.x; c < q_rank; c += 256)
+      cq[t * q_rank + c] = from_f32<T>(to_f32(row[c]) * f * qw[c]);
+  }
+  if (dest == nullptr) return;
+  const T* kv = row + kvoff;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < rank; c += 256) {
+    const float v = to_f32(kv[c]);
+    ss += v * v;
+  }
+  const float f = rsqrtf(la_block_sum(ss, red) / (float)rank + eps);
+  T* out = kcache + (size_t)dest[t] * (rank + rot);
+  for (int c = threadIdx.x; c < rank; c += 256) out[c] = from_f32<T>(to_f32(kv[c]) * f * kw[c]);
+  const float* ang = angles + t * (size_t)rot_dims;          // (cos, sin) pairs: rot_dims floats a token
+  for (int i = threadIdx.x; i < rot / 2 + (rot & 1); i += 256) {
+    const float u = to_f32(kv[rank + 2 * i]);
+    if (2 * i + 1 >= rot) { out[rank + 2 * i] = from_f32<T>(u); continue; }
+    const float v = to_f32(kv[rank + 2 * i + 1]);
+    if (2 * i + 1 < rot_dims) {
+      const float c = ang[2 * i], s = ang[2 * i + 1];
+      out[rank + 2 * i] = from_f32<T>(u * c - v * s);
+      out[rank + 2 * i + 1] = from_f32<T>(v * c + u * s);
+    } else {
+      out[rank + 2 * i] = from_f32<T>(u);
+      out[rank + 2 * i + 1] = from_f32<T>(v);
+    }
+  }
+}
+
+// proj: [nt, stride] rows: the query latent (q_rank) first, the key/value latent (rank) and the
+// shared key part (rot) from column kvoff. cq: [nt, q_rank]. dest null: the step's rows store
+// nothing (the layer reads rows that another layer stored). kcache: [pages, 1, PAGE, rank + rot].
+extern "C" int ta_latent_prepare(hipStream_t stream, int dtype, const void* proj, int stride, int q_rank,
+                                 const float* qw, void* cq, int kvoff, int rank, int rot, int rot_dims,
+                                 const float* kw, float eps, const float* angles, const int* dest,
+                                 void* kcache, int nt) {
+  TA_REQUIRE(nt >= 0 && q_rank >= 0 && rank >= 1 && rot >= 0 && rot_dims >= 0 && rot_dims <= rot && rot_dims % 2 == 0,
+             "ta_latent_prepare: bad sizes nt=%d q_rank=%d rank=%d rot=%d dims=%d", nt, q_rank, rank, rot, rot_dims);
+  TA_REQUIRE(q_rank > 0 || dest != nullptr, "ta_latent_prepare: nothing to do");
+  TA_REQUIRE(dest == nullptr || rot_dims == 0 || angles != nullptr, "ta_latent_prepare: angles are required");
+  if (nt == 0) return 0;
+  if (dtype == TA_F32)
+    latent_prepare_kernel<float><<<nt, 256, 0, stream>>>((const float*)proj, stride, q_rank, qw, (float*)cq, kvoff, rank,
+                                                        rot, rot_dims, kw, eps, angles, dest, (float*)kcache);
+  else if (dtype == TA_BF16)
+    latent_prepare_kernel<bf16_t><<<nt, 256, 0, stream>>>((const bf16_t*)proj, stride, q_rank, qw, (bf16_t*)cq, kvoff,
+                                                         rank, rot, rot_dims, kw, eps, angles, dest, (bf16_t*)kcache);
+  else
+    return ta_fail("ta_latent_prepare: unknown dtype %d", dtype);
+  return ta_check_launch("ta_latent_prepare");
+}
+
+// ------------------------------------------------------------------ rotated query parts
+template <typename T>
+__global__ __launch_bounds__(256) void latent_query_rot_kernel(const T* __restrict__ q, int H, int dn, int rot,
+                                                               int rot_dims, const float* __restrict__ angles,
+                                                               T* __restrict__ qa, int rank) {
+  const size_t t = blockIdx.x;
+  const float* ang = angles + t * (size_t)rot_dims;
+  const int pairs = (rot + 1) / 2;
+  for (int idx = threadIdx.x; idx < H * pairs; idx += 256) {
+    const int h = idx / pairs, i = idx % pairs;
+    const T* src = q + (t * H + h) * (size_t)(dn + rot) + dn;
+    T* dst = qa + (t * H + h) * (size_t)(rank + rot) + rank;
+    const float u = to_f32(src[2 * i]);
+    if (2 * i + 1 >= rot) { dst[2 * i] = from_f32<T>(u); continue; }
+    const float v = to_f32(src[2 * i + 1]);
+    if (2 * i + 1 < rot_dims) {
+      const float c = ang[2 * i], s = ang[2 * i + 1];
+      dst[2 * i] = from_f32<T>(u * c - v * s);
+      dst[2 * i + 1] = from_f32<T>(v * c + u * s);
+    } else {
+      dst[2 * i] = from_f32<T>(u);
+      dst[2 * i + 1] = from_f32<T>(v);
+    }
+  }
+}
+
+// q: [nt, H, dn + rot] (each head: unrotated part, then the part to rotate); qa: [nt, H, rank + rot],
+// whose last rot coordinates per head are written.
+extern "C" int ta_latent_query_rot(hipStream_t stream, int dtype, const void* q, int H, int dn, int rot,
+                                   int rot_dims, const float* angles, void* qa, int rank, int nt) {
+  TA_REQUIRE(nt >= 0 && H >= 1 && dn >= 0 && rot >= 0 && rank >= 1 && rot_dims >= 0 && rot_dims <= rot && rot_dims % 2 == 0,
+             "ta_latent_query_rot: bad sizes");
+  if (nt == 0 || rot == 0) return 0;
+  if (dtype == TA_F32)
+    latent_query_rot_kernel<float><<<nt, 256, 0, stream>>>((const float*)q, H, dn, rot, rot_dims, angles, (float*)qa, rank);
+  else if (dtype == TA_BF16)
+    latent_query_rot_kernel<bf16_t><<<nt, 256, 0, stream>>>((const bf16_t*)q, H, dn, rot, rot_dims, angles, (bf16_t*)qa, rank);
+  else
+    return ta_fail("ta_latent_query_rot: unknown dtype %d", dtype);
+  return ta_check_launch("ta_latent_query_rot");
+}
+
+// ------------------------------------------------------------------ attention
+// A workgroup owns 16 rows, row = (query token, head); 16 lanes share a row. The 32 keys of
+// a chunk sit in LDS once and serve as keys (all D coordinates) and as values (the first
+// `rank`). NACC: output coordinates per lane (rank <= 16 * NACC).
+#define LA_ROWS 16
+#define LA_CHUNK 32
+
+__device__ __forceinline__ float la16_max(float v) {
+#pragma unroll
+  for (int o = 8; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 16));
+  return v;
+}
+__device__ __forceinline__ float la16_sum(float v) {
+#pragma unroll
+  for (int o = 8; o > 0; o >>= 1) v += __shfl_xor(v, o, 16);
+  return v;
+}
+
+template <typename T, int NACC>
+__global__ __launch_bounds__(256) void latent_attention_kernel(
+    const T* __restrict__ qa, T* __restrict__ out, const T* __restrict__ kcache,
+    const int* __restrict__ block_table, int max_blocks, const int* __restrict__ cu_q,
+    const int* __restrict__ pos0, int H, int rank, int rot, float scale, int window,
+    const T* __restrict__ gate, int gate_stride) {
+  extern __shared__ float smem[];
+  const int D = rank + rot, DP = D + 1;
+  const int b = blockIdx.y;
+  const int q0 = cu_q[b], qlen = cu_q[b + 1] - q0;
+  const int nrows = qlen * H;
+  const int row0 = blockIdx.x * LA_ROWS;
+  if (row0 >= nrows) return;
+  const int p0 = pos0[b];
+  const int rloc = threadIdx.x / 16, lane = threadIdx.x % 16;
+  const int row = row0 + rloc;
+  const bool row_ok = row < nrows;
+  const int qi = row_ok ? row / H : 0;
+  const int head = row_ok ? row % H : 0;
+  float* Qs = smem;                          // [LA_ROWS][D]
+  float* Ks = Qs + LA_ROWS * D;              // [LA_CHUNK][D + 1]
+  float* Ps = Ks + LA_CHUNK * DP;            // [LA_ROWS][LA_CHUNK]
+
+  for (int i = threadIdx.x; i < LA_ROWS * D; i += 256) {
+    const int r = i / D, d = i - r * D, rr = row0 + r;
+    Qs[i] = rr < nrows ? to_f32(qa[((size_t)(q0 + rr / H) * H + rr % H) * D + d]) : 0.f;
+  }
+  const int qi_min = row0 / H;
+  const int last_row = (row0 + LA_ROWS - 1 < nrows - 1) ? row0 + LA_ROWS - 1 : nrows - 1;
+  const int tile_end = p0 + last_row / H + 1;                          // exclusive
+  int tile_start = 0;
+  if (window > 0) {
+    tile_start = p0 + qi_min + 1 - window;
+    if (tile_start < 0) tile_start = 0;
+  }
+  const int my_end = p0 + qi + 1;
+  int my_start = 0;
+  if (window > 0) {
+    my_start = my_end - window;
+    if (my_start < 0) my_start = 0;
+  }
+  float acc[NACC];
+#pragma unroll
+  for (int i = 0; i < NACC; ++i) acc[i] = 0.f;
+  float m = -INFINITY, l = 0.f;
+  const int* table = block_table + (size_t)b * max_blocks;
+  for (int c = tile_start / LA_CHUNK; c * LA_CHUNK < tile_end; ++c) {
+    const int key0 = c * LA_CHUNK;
+    const size_t page = (size_t)table[key0 / TA_PAGE];
+    const size_t base = (page * TA_PAGE + key0 % TA_PAGE) * (size_t)D;
+    __syncthreads();                         // the chunk before has been read
+    for (int i = threadIdx.x; i < LA_CHUNK * D; i += 256) {
+      const int k = i / D, d = i - k * D;
+      Ks[k * DP + d] = (key0 + k < tile_end) ? to_f32(kcache[base + i]) : 0.f;
+    }
+    __syncthreads();
+    float s0 = 0.f, s1 = 0.f;
+    {
+      const float* qr = Qs + rloc * D;
+      const float* k0 = Ks + lane * DP;
+      const float* k1 = Ks + (lane + 16) * DP;
+      for (int d = 0; d < D; ++d) {
+        const float qv = qr[d];
+        s0 = fmaf(qv, k0[d], s0);
+        s1 = fmaf(qv, k1[d], s1);
+      }
+    }
+    const int kk0 = key0 + lane, kk1 = kk0 + 16;
+    const bool v0 = row_ok && kk0 >= my_start && kk0 < my_end;
+    const bool v1 = row_ok && kk1 >= my_start && kk1 < my_end;
+    s0 = v0 ? s0 * scale : -INFINITY;
+    s1 = v1 ? s1 * scale : -INFINITY;
+    const float m_new = fmaxf(m, la16_max(fmaxf(s0, s1)));
+    float alpha = 1.f, e0 = 0.f, e1 = 0.f;
+    if (m_new != -INFINITY) {
+      alpha = expf(m - m_new);
+      e0 = v0 ? expf(s0 - m_new) : 0.f;
+      e1 = v1 ? expf(s1 - m_new) : 0.f;
+    }
+    l = l * alpha + la16_sum(e0 + e1);
+    m = m_new;
+#pragma unroll
+    for (int i = 0; i < NACC; ++i) acc[i] *= alpha;
+    Ps[rloc * LA_CHUNK + lane] = e0;
+    Ps[rloc * LA_CHUNK + lane + 16] = e1;
+    __syncthreads();
+    {
+      const float* pr = Ps + rloc * LA_CHUNK;
+      for (int k = 0; k < LA_CHUNK; ++k) {
+        const float p = pr[k];
+        const float* vr = Ks + k * DP + lane;
+#pragma unroll
+        for (int i = 0; i < NACC; ++i)
+          if (16 * i + lane < rank) acc[i] = fmaf(p, vr[16 * i], acc[i]);
+      }
+    }
+  }
+  if (row_ok) {
+    float f = l > 0.f ? 1.0f / l : 0.f;
+    if (gate) {
+      const float g = to_f32(gate[(size_t)(q0 + qi) * gate_stride + head]);
+      f *= 1.0f / (1.0f + expf(-g));
+    }
+    T* o = out + ((size_t)(q0 + qi) * H + head) * rank + lane;
+#pragma unroll
+    for (int i = 0; i < NACC; ++i)
+      if (16 * i + lane < rank) o[16 * i] = from_f32<T>(acc[i] * f);
+  }
+}
+
+template <typename T, int NACC>
+static int latent_attention_run(hipStream_t stream, dim3 g, size_t lds, const void* qa, void* out,
+                                const void* kcache, const int* block_table, int max_blocks, const int* cu_q,
+                                const int* pos0, int H, int rank, int rot, float scale, int window,
+                                const void* gate, int gate_stride) {
+  auto kern = latent_attention_kernel<T, NACC>;
+  if (lds > 64 * 1024) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return ta_fail("ta_latent_attention: %zu bytes of LDS refused (%s)", lds, hipGetErrorString(e));
+  }
+  kern<<<g, 256, lds, stream>>>((const T*)qa, (T*)out, (const T*)kcache, block_table, max_blocks, cu_q, pos0, H,
+                                rank, rot, scale, window, (const T*)gate, gate_stride);
+  return 0;
+}
+
+// qa: [nt, H, rank + rot] wide queries. out: [nt, H, rank]. kcache: one layer,
+// [pages][1][TA_PAGE][rank + rot]. gate (or null): pre-activation of a sigmoid gate per
+// (token, head), element h of a row of gate_stride elements. window <= 0: all earlier keys.
+extern "C" int ta_latent_attention(hipStream_t stream, int dtype, const void* qa, void* out, const void* kcache,
+                                   const int* block_table, int max_blocks, const int* cu_q, const int* pos0,
+                                   int batch, int max_qlen, int H, int rank, int rot, float scale, int window,
+                                   const void* gate, int gate_stride) {
+  TA_REQUIRE(batch >= 0 && batch <= 65535 && max_qlen >= 0 && H >= 1, "ta_latent_attention: bad batch=%d max_qlen=%d heads=%d", batch, max_qlen, H);
+  TA_REQUIRE(rank >= 1 && rank <= 512 && rot >= 0 && rot <= 512, "ta_latent_attention: latent of %d / rotated part of %d outside [1, 512] / [0, 512]", rank, rot);
+  TA_REQUIRE(max_blocks > 0, "ta_latent_attention: empty block table");
+  TA_REQUIRE(gate == nullptr || gate_stride >= H, "ta_latent_attention: gate rows too short");
+  if (batch == 0 || max_qlen == 0) return 0;
+  const long long tiles = ((long long)max_qlen * H + LA_ROWS - 1) / LA_ROWS;
+  TA_REQUIRE(tiles <= 2147483647ll, "ta_latent_attention: too many rows");
+  dim3 g((unsigned)tiles, batch);
+  const int D = rank + rot;
+  const size_t lds = (size_t)(LA_ROWS * D + LA_CHUNK * (D + 1) + LA_ROWS * LA_CHUNK) * sizeof(float);
+  TA_REQUIRE(lds <= 160 * 1024, "ta_latent_attention: rows of %d do not fit the LDS", D);
+  int rc;
+#define LA_RUN(T)                                                                                              \
+  (rank <= 128 ? latent_attention_run<T, 8>(stream, g, lds, qa, out, kcache, block_table, max_blocks, cu_q, pos0, H, rank, rot, scale, window, gate, gate_stride)   \
+   : rank <= 256 ? latent_attention_run<T, 16>(stream, g, lds, qa, out, kcache, block_table, max_blocks, cu_q, pos0, H, rank, rot, scale, window, gate, gate_stride) \
+                 : latent_attention_run<T, 32>(stream, g, lds, qa, out, kcache, block_table, max_blocks, cu_q, pos0, H, rank, rot, scale, window, gate, gate_stride))
+  if (dtype == TA_F32) rc = LA_RUN(float);
+  else if (dtype == TA_BF16) rc = LA_RUN(bf16_t);
+  else return ta_fail("ta_latent_attention: unknown dtype %d", dtype);
+#undef LA_RUN
+  if (rc) return rc;
+  return ta_check_launch("ta_latent_attention");
+}

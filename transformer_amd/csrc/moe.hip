@@ -1,0 +1,356 @@
+// Routed feed-forward: every token is sent to `top` of E small feed-forward layers.
+//
+//   moe_route   : scores = f(router logits) per token (sigmoid, or softmax over the experts),
+//                 the `top` largest (lowest index among equals), optionally renormalised
+//   moe_plan    : the (token, choice) pairs ordered by expert: each expert's pairs take a run
+//                 of rows that starts on a multiple of 16, so a tile of 16 rows belongs to one
+//                 expert; the row count is bounded by pairs + 15 * E whatever the routing is,
+//                 so a step's launches do not depend on the data
+//   moe_gather  : the ordered rows of activations, each times its pair's weight when the weight
+//                 acts on the expert's input
+//   moe_gemm    : C[rows of a tile] = A[rows] * W[expert of the tile]^T for all tiles, with an
+//                 optional activation; float32 chains on the vector ALU, or the matrix cores
+//                 (v_mfma_f32_16x16x32_bf16) for bfloat16
+//   moe_combine : delta[t] = sum of the token's pairs' rows (times the weight when it acts on
+//                 the output) + sigmoid(shared gate) * the shared expert's rows
+//
+// Router scores, weights and all sums are float32.
+#include "common.h"
+
+#define MOE_TILE 16
+
+// ------------------------------------------------------------------ routing
+// logits: [nt, ld] float32, the first E columns of a row are the router's. mode 0: sigmoid
+// scores; 1: softmax over the experts. renorm: the chosen weights are divided by their sum.
+__global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__ logits, int ld, int E, int top,
+                                                       int mode, int renorm, int* __restrict__ chosen,
+                                                       float* __restrict__ weight) {
+  extern __shared__ float sc[];           // [E]
+  const size_t t = blockIdx.x;
+  const int lane = threadIdx.x;
+  float mx = -INFINITY;
+  for (int e = lane; e < E; e += 64) mx = fmaxf(mx, logits[t * ld + e]);
+  mx = wave_max(mx);
+  float sum = 0.f;
+  for (int e = lane; e < E; e += 64) {
+    const float z = logits[t * ld + e];
+    const float s = mode == 0 ? 1.0f / (1.0f + expf(-z)) : expf(z - mx);
+    sc[e] = s;
+    sum += s;
+  }
+  sum = wave_sum(sum);
+  __syncthreads();
+  float total = 0.f;
+  for (int j = 0; j < top; ++j) {
+    float best = -INFINITY;
+    int at = 0x7fffffff;
+    for (int e = lane; e < E; e += 64) {
+      const float s = sc[e];
+      if (s > best) { best = s; at = e; }       // ascending e: the lowest index among equals
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ob = __shfl_xor(best, o, TA_WAVE);
+      const int oa = __shfl_xor(at, o, TA_WAVE);
+      if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; }
+    }
+    const float w = mode == 0 ? best : best / sum;
+    if (lane == 0) {
+      chosen[t * top + j] = at;
+      weight[t * top + j] = w;
+    }
+    total += w;
+    __syncthreads();
+    if (lane == 0) sc[at] = -INFINITY;
+    __syncthreads();
+  }
+  if (renorm) {
+    __syncthreads();
+    for (int j = lane; j < top; j += 64) weight[t * top + j] /= total;
+  }
+}
+
+extern "C" int ta_moe_route(hipStream_t stream, const float* logits, int ld, int nt, int E, int top, int mode,
+                            int renorm, int* chosen, float* weight) {
+  TA_REQUIRE(nt >= 0 && E >= 1 && E <= 8192 && top >= 1 && top <= E && ld >= E && (mode == 0 || mode == 1),
+             "ta_moe_route: bad sizes nt=%d experts=%d top=%d ld=%d", nt, E, top, ld);
+  if (nt == 0) return 0;
+  moe_route_kernel<<<nt, 64, (size_t)E * sizeof(float), stream>>>(logits, ld, E, top, mode, renorm, chosen, weight);
+  return ta_check_launch("ta_moe_route");
+}
+
+// ------------------------------------------------------------------ ordering the pairs by expert
+// One workgroup. row_pair: [max_rows] pair index of every ordered row, -1 for a row that only
+// fills a tile; tile_expert: [max_rows / 16], -1 for a tile past the last; pair_row: [pairs].
+__global__ __launch_bounds__(1024) void moe_plan_kernel(const int* __restrict__ chosen, int pairs, int E,
+                                                        int max_rows, int* __restrict__ row_pair,
+                                                        int* __restrict__ tile_expert, int* __restrict__ pair_row) {
+  extern __shared__ int sh[];             // count [E], start [E + 1]
+  int* count = sh;
+  int* start = sh + E;
+  for (int e = threadIdx.x; e < E; e += 1024) count[e] = 0;
+  for (int i = threadIdx.x; i < max_rows; i += 1024) row_pair[i] = -1;
+  __syncthreads();
+  for (int i = threadIdx.x; i < pairs; i += 1024) atomicAdd(&count[chosen[i]], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int at = 0;
+    for (int e = 0; e < E; ++e) {
+      start[e] = at;
+      at += (count[e] + MOE_TILE - 1) / MOE_TILE * MOE_TILE;
+    }
+    start[E] = at;
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < max_rows / MOE_TILE; i += 1024) {
+    const int r = i * MOE_TILE;
+    int e = -1;
+    if (r < start[E]) {                   // the last expert whose run starts at or before r
+      int lo = 0, hi = E - 1;
+      while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (start[mid] <= r) lo = mid; else hi = mid - 1;
+      }
+      e = lo;
+    }
+    tile_expert[i] = e;
+  }
+  for (int e = threadIdx.x; e < E; e += 1024) count[e] = 0;
+  __syncthreads();
+  // the order of an expert's rows among themselves does not matter: every row is computed alone
+  for (int i = threadIdx.x; i < pairs; i += 1024) {
+    const int e = chosen[i];
+    const int r = start[e] + atomicAdd(&count[e], 1);
+    row_pair[r] = i;
+    pair_row[i] = r;
+  }
+}
+
+extern "C" int ta_moe_max_rows(int pairs, int E) {
+  const long long n = (long long)pairs + (long long)(MOE_TILE - 1) * E;
+  const long long r = (n + MOE_TILE - 1) / MOE_TILE * MOE_TILE;
+  return r > 2147483647ll ? -1 : (int)r;
+}
+
+extern "C" int ta_moe_plan(hipStream_t stream, const int* chosen, int pairs, int E, int max_rows, int* row_pair,
+                           int* tile_expert, int* pair_row) {
+  TA_REQUIRE(pairs >= 0 && E >= 1 && E <= 8192, "ta_moe_plan: bad sizes pairs=%d experts=%d", pairs, E);
+  TA_REQUIRE(max_rows == ta_moe_max_rows(pairs, E), "ta_moe_plan: %d rows for %d pairs of %d experts", max_rows, pairs, E);
+  moe_plan_kernel<<<1, 1024, (size_t)(2 * E + 1) * sizeof(int), stream>>>(chosen, pairs, E, max_rows, row_pair,
+                                                                        tile_expert, pair_row);
+  return ta_check_launch("ta_moe_plan");
+}
+
+// ------------------------------------------------------------------ gathering the rows
+template <typename T>
+__global__ __launch_bounds__(256) void moe_gather_kernel(const T* __restrict__ h, int d, int top,
+                                                         const int* __restrict__ row_pair,
+                                                         const float* __restrict__ weight, T* __restrict__ out) {
+  const size_t r = blockIdx.x;
+  const int pair = row_pair[r];
+  T* dst = out + r * d;
+  if (pair < 0) {
+    for (int c = threadIdx.x; c < d; c += 256) dst[c] = from_f32<T>(0.f);
+    return;
+  }
+  const T* src = h + (size_t)(pair / top) * d;
+  if (weight) {
+    const float w = weight[pair];
+    for (int c = threadIdx.x; c < d; c += 256) dst[c] = from_f32<T>(to_f32(src[c]) * w);
+  } else {
+    for (int c = threadIdx.x; c < d; c += 256) dst[c] = src[c];
+  }
+}
+
+// out[r] = h[token of row r] (* weight of its pair; weight null: as it is); filling rows are zero.
+extern "C" int ta_moe_gather(hipStream_t stream, int dtype, const void* h, int d, int top, const int* row_pair,
+                             const float* weight, void* out, int max_rows) {
+  TA_REQUIRE(d > 0 && top >= 1 && max_rows >= 0, "ta_moe_gather: bad sizes");
+  if (max_rows == 0) return 0;
+  if (dtype == TA_F32)
+    moe_gather_kernel<float><<<max_rows, 256, 0, stream>>>((const float*)h, d, top, row_pair, weight, (float*)out);
+  else if (dtype == TA_BF16)
+    moe_gather_kernel<bf16_t><<<max_rows, 256, 0, stream>>>((const bf16_t*)h, d, top, row_pair, weight, (bf16_t*)out);
+  else
+    return ta_fail("ta_moe_gather: unknown dtype %d", dtype);
+  return ta_check_launch("ta_moe_gather");
+}
+
+// ------------------------------------------------------------------ the experts' products
+__device__ __forceinline__ float moe_act(int act, float z) {
+  switch (act) {
+    case 1: return 0.5f * z * (1.0f + erff(z * 0.7071067811865476f));
+    case 2: return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+    case 3: { const float r = fmaxf(z, 0.f); return r * r; }
+    case 4: return z / (1.0f + expf(-z));
+    default: return z;
+  }
+}
+
+// float32 chains: a workgroup owns a tile of 16 rows and 64 columns; a thread 1 row x 4 columns.
+// Every element is one ascending-k chain of fused multiply-adds.
+template <typename T, typename TC>
+__global__ __launch_bounds__(256) void moe_gemm_fma_kernel(const T* __restrict__ A, const T* __restrict__ W,
+                                                           const int* __restrict__ tile_expert, TC* __restrict__ C,
+                                                           int N, int K, int act) {
+  __shared__ float As[16][MOE_TILE + 1];
+  __shared__ float Ws[16][64 + 1];
+  const int e = tile_expert[blockIdx.y];
+  if (e < 0) return;
+  const size_t r0 = (size_t)blockIdx.y * MOE_TILE;
+  const int n0 = blockIdx.x * 64;
+  const T* We = W + (size_t)e * N * K;
+  const int tr = threadIdx.x / 16, tc = threadIdx.x % 16;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < K; k0 += 16) {
+    {
+      const int r = threadIdx.x / 16, k = k0 + threadIdx.x % 16;
+      As[threadIdx.x % 16][r] = k < K ? to_f32(A[(r0 + r) * K + k]) : 0.f;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int idx = threadIdx.x + 256 * i, n = idx / 16, k = k0 + idx % 16;
+      Ws[idx % 16][n] = (n0 + n < N && k < K) ? to_f32(We[(size_t)(n0 + n) * K + k]) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < 16; ++kk) {
+      const float a = As[kk][tr];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[j] = fmaf(a, Ws[kk][tc * 4 + j], acc[j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int n = n0 + tc * 4 + j;
+    if (n < N) C[(r0 + tr) * N + n] = from_f32<TC>(moe_act(act, acc[j]));
+  }
+}
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 moe_bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float moe_floatx4;
+typedef uint32_t moe_u32x4 __attribute__((ext_vector_type(4)));
+union MoeFrag {
+  moe_bf16x8 v;
+  moe_u32x4 q;
+};
+
+// Matrix cores: a workgroup of 4 waves owns a tile of 16 rows; a wave 64 columns (four 16 x 16
+// tiles) and walks K in steps of 32: a lane holds 8 consecutive k of row (lane % 16) of its
+// operand. K % 8 == 0; the last step's missing k are zero.
+template <typename TC>
+__global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W,
+                                                            const int* __restrict__ tile_expert,
+                                                            TC* __restrict__ C, int N, int K, int act) {
+  const int e = tile_expert[blockIdx.y];
+  if (e < 0) return;
+  const size_t r0 = (size_t)blockIdx.y * MOE_TILE;
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  const int n0 = (blockIdx.x * 4 + wave) * 64;
+  if (n0 >= N) return;
+  const bf16_t* We = W + (size_t)e * N * K;
+  const int r = lane % 16, kb = lane / 16;
+  const bf16_t* arow = A + (r0 + r) * K + kb * 8;
+  const bf16_t* wrow[4];
+  bool wok[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    const int n = n0 + 16 * t + r;
+    wok[t] = n < N;
+    wrow[t] = We + (size_t)(wok[t] ? n : 0) * K + kb * 8;
+  }
+  moe_floatx4 acc[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) acc[t] = moe_floatx4{0.f, 0.f, 0.f, 0.f};
+  const moe_u32x4 zero = {0, 0, 0, 0};
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    const bool kok = k0 + kb * 8 < K;
+    MoeFrag af;
+    af.q = kok ? *reinterpret_cast<const moe_u32x4*>(arow + k0) : zero;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      MoeFrag wf;
+      wf.q = (kok && wok[t]) ? *reinterpret_cast<const moe_u32x4*>(wrow[t] + k0) : zero;
+      // register j of a lane: W row 4 * (lane / 16) + j of the tile, activation row lane % 16
+      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf.v, af.v, acc[t], 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + 16 * t + 4 * kb + j;
+      if (n < N) C[(r0 + r) * N + n] = from_f32<TC>(moe_act(act, acc[t][j]));
+    }
+}
+
+// A: [max_rows, K] ordered rows; W: [E, N, K]; C: [max_rows, N], float32 or the type of A;
+// act: 0 none, 1 gelu, 2 gelu (tanh), 3 relu squared, 4 silu. Tiles past the last expert's
+// rows are skipped and their rows of C keep what they held.
+extern "C" int ta_moe_gemm(hipStream_t stream, int dtype, int out_dtype, const void* A, const void* W,
+                           const int* tile_expert, void* C, int max_rows, int N, int K, int act) {
+  TA_REQUIRE(max_rows >= 0 && max_rows % MOE_TILE == 0 && N > 0 && K > 0 && act >= 0 && act <= 4,
+             "ta_moe_gemm: bad sizes rows=%d N=%d K=%d act=%d", max_rows, N, K, act);
+  if (max_rows == 0) return 0;
+  const int tiles = max_rows / MOE_TILE;
+  if (dtype == TA_BF16 && K % 8 == 0) {
+    dim3 g((N + 255) / 256, tiles);
+    if (out_dtype == TA_BF16)
+      moe_gemm_mfma_kernel<bf16_t><<<g, 256, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, tile_expert, (bf16_t*)C, N, K, act);
+    else if (out_dtype == TA_F32)
+      moe_gemm_mfma_kernel<float><<<g, 256, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, tile_expert, (float*)C, N, K, act);
+    else
+      return ta_fail("ta_moe_gemm: unknown output type %d", out_dtype);
+    return ta_check_launch("ta_moe_gemm");
+  }
+  dim3 g((N + 63) / 64, tiles);
+  if (dtype == TA_F32 && out_dtype == TA_F32)
+    moe_gemm_fma_kernel<float, float><<<g, 256, 0, stream>>>((const float*)A, (const float*)W, tile_expert, (float*)C, N, K, act);
+  else if (dtype == TA_BF16 && out_dtype == TA_BF16)
+    moe_gemm_fma_kernel<bf16_t, bf16_t><<<g, 256, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, tile_expert, (bf16_t*)C, N, K, act);
+  else if (dtype == TA_BF16 && out_dtype == TA_F32)
+    moe_gemm_fma_kernel<bf16_t, float><<<g, 256, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, tile_expert, (float*)C, N, K, act);
+  else
+    return ta_fail("ta_moe_gemm: unsupported types %d -> %d", dtype, out_dtype);
+  return ta_check_launch("ta_moe_gemm");
+}
+
+// ------------------------------------------------------------------ putting the rows back
+__global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ rows, int d, int top,
+                                                          const int* __restrict__ pair_row,
+                                                          const float* __restrict__ weight,
+                                                          const float* __restrict__ shared, int planes, size_t plane,
+                                                          const float* __restrict__ shared_gate, int gate_ld,
+                                                          float* __restrict__ delta) {
+  const size_t t = blockIdx.x;
+  float sg = 1.f;
+  if (shared && shared_gate) sg = 1.0f / (1.0f + expf(-shared_gate[t * gate_ld]));
+  for (int c = threadIdx.x; c < d; c += 256) {
+    float s = 0.f;
+    for (int j = 0; j < top; ++j) {
+      const float v = rows[(size_t)pair_row[t * top + j] * d + c];
+      s += weight ? v * weight[t * top + j] : v;
+    }
+    if (shared) {
+      float v = shared[t * d + c];
+      for (int p = 1; p < planes; ++p) v += shared[t * d + c + p * plane];
+      s += sg * v;
+    }
+    delta[t * d + c] = s;
+  }
+}
+
+// rows: [max_rows, d] float32, the experts' results in the planned order. weight: null when it
+// has acted on the inputs. shared (or null): [planes, nt, d] float32 planes that add up to the
+// shared expert's result; shared_gate (or null): its gate's pre-activation, one number per
+// token, element 0 of a row of gate_ld float32. delta: [nt, d] float32.
+extern "C" int ta_moe_combine(hipStream_t stream, const float* rows, int d, int top, const int* pair_row,
+                              const float* weight, const float* shared, int planes, long long plane,
+                              const float* shared_gate, int gate_ld, float* delta, int nt) {
+  TA_REQUIRE(nt >= 0 && d > 0 && top >= 1 && planes >= 1 && planes <= TA_MAX_PLANES, "ta_moe_combine: bad sizes");
+  if (nt == 0) return 0;
+  moe_combine_kernel<<<nt, 256, 0, stream>>>(rows, d, top, pair_row, weight, shared, planes, (size_t)plane,
+                                             shared_gate, gate_ld, delta);
+  return ta_check_launch("ta_moe_combine");
+}

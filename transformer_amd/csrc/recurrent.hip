@@ -523,15 +523,23 @@ extern "C" int ta_rglru_scan(hipStream_t stream, int dtype, const void* yx, int 
 template <typename T, typename TW>
 __global__ __launch_bounds__(256) void gla_decay_kernel(const T* __restrict__ proj, int stride, int aoff, int rank,
                                                         const TW* __restrict__ a2, const float* __restrict__ a2b,
-                                                        float inv_tau, int n, float* __restrict__ alpha) {
+                                                        float inv_tau, int n, float* __restrict__ alpha,
+                                                        int mode) {
   extern __shared__ float low[];          // [rank]
   const size_t t = blockIdx.x;
-  for (int r = threadIdx.x; r < rank; r += 256) low[r] = to_f32(proj[t * stride + aoff + r]);
+  for (int r = threadIdx.x; r < rank; r += 256) {
+    const float v = to_f32(proj[t * stride + aoff + r]);
+    low[r] = mode == 1 ? tanhf(v) : v;
+  }
   __syncthreads();
   for (int c = blockIdx.y * 256 + threadIdx.x; c < n; c += gridDim.y * 256) {
     const TW* w = a2 + (size_t)c * rank;
     float z = a2b[c];
     for (int r = 0; r < rank; ++r) z = fmaf(to_f32(w[r]), low[r], z);
+    if (mode == 1) {                      // the double-exponential decay: exp(-exp(z)), z from tanh(low)
+      alpha[t * n + c] = expf(-expf(z));
+      continue;
+    }
     // sigmoid(z)^(1/tau) = exp(log sigmoid(z) / tau), log sigmoid(z) = min(z, 0) - log1p(exp(-|z|))
     alpha[t * n + c] = expf((fminf(z, 0.f) - log1pf(expf(-fabsf(z)))) * inv_tau);
   }
@@ -554,11 +562,14 @@ struct GlaOperands {  // what one thread brings in for a chunk
   float q[GLA_TC * GLA_RT / 256], k[GLA_TC * GLA_RT / 256], a[GLA_TC * GLA_RT / 256], v[GLA_TC * GLA_CT / 256];
 };
 
-template <typename T, int GLA_TC>
+// BONUS: the readout comes BEFORE the update and gives the current token a weight of its own,
+// o_t = (S_{t-1} + diag(bonus) k_t v_t^T)^T q_t, then S_t = diag(alpha_t) S_{t-1} + k_t v_t^T.
+template <typename T, int GLA_TC, bool BONUS>
 __global__ __launch_bounds__(256) void gla_recurrent_kernel(
     const T* __restrict__ proj, int stride, int qoff, int koff, int voff, const float* __restrict__ alpha,
     float qscale, float* __restrict__ state, const int* __restrict__ cu_q, const int* __restrict__ slots,
-    int H, int dk, int dv, int col_tiles, size_t plane, float* __restrict__ o_out) {
+    int H, int dk, int dv, int col_tiles, size_t plane, float* __restrict__ o_out,
+    const float* __restrict__ bonus) {
   __shared__ float sq[GLA_TC][GLA_RT], sk[GLA_TC][GLA_RT], sa[GLA_TC][GLA_RT];
   __shared__ float sv[GLA_TC][GLA_CT];
   __shared__ float part[GLA_TC][4][GLA_CT];
@@ -579,6 +590,14 @@ __global__ __launch_bounds__(256) void gla_recurrent_kernel(
       const int i = row0 + rg * 4 + r, j = col0 + cg * 2 + c;
       S[r][c] = (i < dk && j < dv) ? st[(size_t)i * dv + j] : 0.f;
     }
+  float bu[4] = {0.f, 0.f, 0.f, 0.f};
+  if (BONUS) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int i = row0 + rg * 4 + r;
+      bu[r] = i < dk ? bonus[h * dk + i] : 0.f;
+    }
+  }
   // Loads are asked for two chunks ahead (a trip to memory takes longer than a chunk's
   // arithmetic); a position that is not there reads a harmless address and is replaced.
   auto fetch = [&](GlaOperands<GLA_TC>& o, int t0) {
@@ -635,10 +654,18 @@ __global__ __launch_bounds__(256) void gla_recurrent_kernel(
         float a0 = 0.f, a1 = 0.f;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          S[r][0] = fmaf(as[r], S[r][0], ks[r] * v2.x);
-          S[r][1] = fmaf(as[r], S[r][1], ks[r] * v2.y);
-          a0 = fmaf(S[r][0], qs[r], a0);
-          a1 = fmaf(S[r][1], qs[r], a1);
+          if (BONUS) {
+            const float kv0 = ks[r] * v2.x, kv1 = ks[r] * v2.y;
+            a0 = fmaf(fmaf(bu[r], kv0, S[r][0]), qs[r], a0);
+            a1 = fmaf(fmaf(bu[r], kv1, S[r][1]), qs[r], a1);
+            S[r][0] = fmaf(as[r], S[r][0], kv0);
+            S[r][1] = fmaf(as[r], S[r][1], kv1);
+          } else {
+            S[r][0] = fmaf(as[r], S[r][0], ks[r] * v2.x);
+            S[r][1] = fmaf(as[r], S[r][1], ks[r] * v2.y);
+            a0 = fmaf(S[r][0], qs[r], a0);
+            a1 = fmaf(S[r][1], qs[r], a1);
+          }
         }
         p0[u] = a0;
         p1[u] = a1;
@@ -687,11 +714,11 @@ extern "C" int ta_gla_row_parts(int dk) { return (dk + GLA_RT - 1) / GLA_RT; }
 // low-rank decay input (rank) at aoff. a2: [H*dk, rank], a2b [H*dk]. alpha: scratch [nt, H*dk]
 // float32. state: [slots, H, dk, dv] float32. o_out: [ta_gla_row_parts(dk), nt, H, dv] float32,
 // planes that add up to the readout (not yet normalised).
-extern "C" int ta_gla_recurrent(hipStream_t stream, int dtype, int wdtype, const void* proj, int stride,
-                                int qoff, int koff, int voff, int aoff, int rank, const void* a2,
-                                const float* a2b, float inv_tau, float qscale, float* alpha, float* state,
-                                const int* cu_q, const int* slots, int batch, int nt, int H, int dk, int dv,
-                                float* o_out) {
+static int gla_recurrent_launch(hipStream_t stream, int dtype, int wdtype, const void* proj, int stride,
+                                int qoff, int koff, int voff, const void* low, int low_stride, int aoff, int rank,
+                                const void* a2, const float* a2b, float inv_tau, float qscale, float* alpha,
+                                float* state, const int* cu_q, const int* slots, int batch, int nt, int H, int dk,
+                                int dv, float* o_out, int mode, const float* bonus) {
   TA_REQUIRE(batch > 0 && batch <= 65535 && H > 0 && H <= 65535 && nt >= batch,
              "ta_gla_recurrent: bad batch %d / heads %d / tokens %d", batch, H, nt);
   TA_REQUIRE(dk >= 1 && dv >= 1 && rank >= 1 && rank <= 8192, "ta_gla_recurrent: bad widths %d / %d / %d", dk, dv, rank);
@@ -701,7 +728,7 @@ extern "C" int ta_gla_recurrent(hipStream_t stream, int dtype, int wdtype, const
   dim3 gd(nt, (n + 255) / 256 < 64 ? (n + 255) / 256 : 64);
   const size_t lds = (size_t)rank * sizeof(float);
 #define GLA_DECAY(T, TW) \
-  gla_decay_kernel<T, TW><<<gd, 256, lds, stream>>>((const T*)proj, stride, aoff, rank, (const TW*)a2, a2b, inv_tau, n, alpha)
+  gla_decay_kernel<T, TW><<<gd, 256, lds, stream>>>((const T*)low, low_stride, aoff, rank, (const TW*)a2, a2b, inv_tau, n, alpha, mode)
   if (dtype == TA_F32 && wdtype == TA_F32) GLA_DECAY(float, float);
   else if (dtype == TA_BF16 && wdtype == TA_BF16) GLA_DECAY(bf16_t, bf16_t);
   else if (dtype == TA_BF16 && wdtype == TA_F32) GLA_DECAY(bf16_t, float);
@@ -710,16 +737,46 @@ extern "C" int ta_gla_recurrent(hipStream_t stream, int dtype, int wdtype, const
   dim3 g(batch, H, parts * tiles);
   const size_t plane = (size_t)nt * H * dv;
   const bool few = nt <= 8 * batch;         // at most 8 tokens a sequence on average: short chunks
-#define GLA_RUN(T, TC)                                                                                   \
-  gla_recurrent_kernel<T, TC><<<g, 256, 0, stream>>>((const T*)proj, stride, qoff, koff, voff, alpha, qscale, \
-                                                     state, cu_q, slots, H, dk, dv, tiles, plane, o_out)
-  if (dtype == TA_F32) {
-    if (few) GLA_RUN(float, 8); else GLA_RUN(float, 32);
+#define GLA_RUN(T, TC, B)                                                                                   \
+  gla_recurrent_kernel<T, TC, B><<<g, 256, 0, stream>>>((const T*)proj, stride, qoff, koff, voff, alpha, qscale, \
+                                                        state, cu_q, slots, H, dk, dv, tiles, plane, o_out, bonus)
+  if (bonus) {
+    if (dtype == TA_F32) {
+      if (few) GLA_RUN(float, 8, true); else GLA_RUN(float, 32, true);
+    } else {
+      if (few) GLA_RUN(bf16_t, 8, true); else GLA_RUN(bf16_t, 32, true);
+    }
+  } else if (dtype == TA_F32) {
+    if (few) GLA_RUN(float, 8, false); else GLA_RUN(float, 32, false);
   } else {
-    if (few) GLA_RUN(bf16_t, 8); else GLA_RUN(bf16_t, 32);
+    if (few) GLA_RUN(bf16_t, 8, false); else GLA_RUN(bf16_t, 32, false);
   }
 #undef GLA_RUN
   return ta_check_launch("ta_gla_recurrent");
+}
+
+extern "C" int ta_gla_recurrent(hipStream_t stream, int dtype, int wdtype, const void* proj, int stride,
+                                int qoff, int koff, int voff, int aoff, int rank, const void* a2,
+                                const float* a2b, float inv_tau, float qscale, float* alpha, float* state,
+                                const int* cu_q, const int* slots, int batch, int nt, int H, int dk, int dv,
+                                float* o_out) {
+  return gla_recurrent_launch(stream, dtype, wdtype, proj, stride, qoff, koff, voff, proj, stride, aoff, rank, a2,
+                              a2b, inv_tau, qscale, alpha, state, cu_q, slots, batch, nt, H, dk, dv, o_out, 0,
+                              nullptr);
+}
+
+// The recurrence with the readout before the update and a bonus for the current token (see
+// BONUS above) and the decay exp(-exp(a2 tanh(low) + a2b)) per key channel. q, k, v sit at
+// element offsets qoff, koff, voff of ``proj`` with ``stride`` elements between tokens (three
+// planes of one buffer, or three column ranges of its rows); low: [nt, rank] rows of their own.
+extern "C" int ta_wkv_recurrent(hipStream_t stream, int dtype, int wdtype, const void* proj, int stride,
+                                int qoff, int koff, int voff, const void* low, int low_stride, int rank,
+                                const void* a2, const float* a2b, const float* bonus, float* alpha,
+                                float* state, const int* cu_q, const int* slots, int batch, int nt, int H,
+                                int dk, int dv, float* o_out) {
+  TA_REQUIRE(bonus != nullptr, "ta_wkv_recurrent: the bonus is required");
+  return gla_recurrent_launch(stream, dtype, wdtype, proj, stride, qoff, koff, voff, low, low_stride, 0, rank, a2,
+                              a2b, 1.0f, 1.0f, alpha, state, cu_q, slots, batch, nt, H, dk, dv, o_out, 1, bonus);
 }
 
 // ------------------------------------------------------------------ gla: head norm and output gate
@@ -727,7 +784,7 @@ template <typename T>
 __global__ __launch_bounds__(64) void gla_out_kernel(const float* __restrict__ o, int parts, size_t plane,
                                                      const T* __restrict__ proj,
                                                      int stride, int goff, const float* __restrict__ w,
-                                                     float eps, int H, int dv, T* __restrict__ out) {
+                                                     int wstride, float eps, int H, int dv, T* __restrict__ out) {
   extern __shared__ float row[];          // [dv]
   const size_t t = blockIdx.x;
   const int h = blockIdx.y;
@@ -742,23 +799,31 @@ __global__ __launch_bounds__(64) void gla_out_kernel(const float* __restrict__ o
   const float f = rsqrtf(wave_sum(ss) / (float)dv + eps);
   for (int c = threadIdx.x; c < dv; c += 64) {
     const float g = to_f32(proj[t * stride + goff + h * dv + c]);
-    out[t * (size_t)(H * dv) + h * dv + c] = from_f32<T>(row[c] * f * w[c] * (g / (1.0f + expf(-g))));
+    out[t * (size_t)(H * dv) + h * dv + c] = from_f32<T>(row[c] * f * w[h * wstride + c] * (g / (1.0f + expf(-g))));
   }
 }
 
 // o: [parts, nt, H, dv] float32 planes that add up to the readout; the gate's pre-activation sits
-// at column goff of proj; w [dv]; out [nt, H*dv] = rms_norm(o per head) * w * silu(gate).
-extern "C" int ta_gla_out(hipStream_t stream, int dtype, const float* o, int parts, const void* proj, int stride,
-                          int goff, const float* w, float eps, int nt, int H, int dv, void* out) {
+// at element goff of proj, ``stride`` elements between tokens; w [dv] shared by the heads
+// (wstride 0) or [H, dv] (wstride dv); out [nt, H*dv] = rms_norm(o per head) * w * silu(gate).
+extern "C" int ta_gla_out_w(hipStream_t stream, int dtype, const float* o, int parts, const void* proj, int stride,
+                            long long goff, const float* w, int wstride, float eps, int nt, int H, int dv,
+                            void* out) {
   TA_REQUIRE(nt >= 0 && H > 0 && H <= 65535 && dv > 0 && dv <= 15000 && parts >= 1, "ta_gla_out: bad sizes");
+  TA_REQUIRE(wstride == 0 || wstride == dv, "ta_gla_out: weight rows of %d for heads of %d", wstride, dv);
   if (nt == 0) return 0;
   dim3 g(nt, H);
   const size_t plane = (size_t)nt * H * dv, lds = (size_t)dv * sizeof(float);
   if (dtype == TA_F32)
-    gla_out_kernel<float><<<g, 64, lds, stream>>>(o, parts, plane, (const float*)proj, stride, goff, w, eps, H, dv, (float*)out);
+    gla_out_kernel<float><<<g, 64, lds, stream>>>(o, parts, plane, (const float*)proj + goff, stride, 0, w, wstride, eps, H, dv, (float*)out);
   else if (dtype == TA_BF16)
-    gla_out_kernel<bf16_t><<<g, 64, lds, stream>>>(o, parts, plane, (const bf16_t*)proj, stride, goff, w, eps, H, dv, (bf16_t*)out);
+    gla_out_kernel<bf16_t><<<g, 64, lds, stream>>>(o, parts, plane, (const bf16_t*)proj + goff, stride, 0, w, wstride, eps, H, dv, (bf16_t*)out);
   else
     return ta_fail("ta_gla_out: unknown dtype %d", dtype);
   return ta_check_launch("ta_gla_out");
+}
+
+extern "C" int ta_gla_out(hipStream_t stream, int dtype, const float* o, int parts, const void* proj, int stride,
+                          int goff, const float* w, float eps, int nt, int H, int dv, void* out) {
+  return ta_gla_out_w(stream, dtype, o, parts, proj, stride, goff, w, 0, eps, nt, H, dv, out);
 }

@@ -1,0 +1,119 @@
+// Kernels of blocks that norm a sublayer's RESULT before it joins the residual stream, and
+// of the small things such blocks hang on the stream:
+//
+//   postnorm_add     : x += rms_norm(delta) * w   (w = the output norm's weight times the
+//                      layer scale), optionally followed in the same pass by a copy of the
+//                      new row in the engine's type and by the NEXT norm of the stream,
+//                      out = rms_norm(x) * w_next, so that a row is read and written once
+//   activation       : out = act(in) (* rows of a float32 side table), act one of gelu (erf),
+//                      gelu (tanh), relu squared, silu
+//
+// All sums, norms and the stream itself are float32; one workgroup owns a row.
+#include "common.h"
+
+__device__ __forceinline__ float block_sum4(float v, float* red) {
+  v = wave_sum(v);
+  const int w = threadIdx.x / TA_WAVE;
+  __syncthreads();
+  if (threadIdx.x % TA_WAVE == 0) red[w] = v;
+  __syncthreads();
+  float s = 0.f;
+  for (int i = 0; i < (int)(blockDim.x / TA_WAVE); ++i) s += red[i];
+  return s;
+}
+
+template <typename TO>
+__global__ __launch_bounds__(256) void postnorm_add_kernel(
+    float* __restrict__ x, const float* __restrict__ delta, int planes, size_t plane,
+    const float* __restrict__ w, float eps, TO* __restrict__ xcast, const float* __restrict__ w_next,
+    float eps_next, TO* __restrict__ out, int d) {
+  extern __shared__ float row[];          // [d]
+  __shared__ float red[4];
+  const size_t base = (size_t)blockIdx.x * d;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < d; c += 256) {
+    float s = delta[base + c];
+    for (int p = 1; p < planes; ++p) s += delta[base + c + p * plane];
+    row[c] = s;
+    ss += s * s;
+  }
+  const float f = rsqrtf(block_sum4(ss, red) / (float)d + eps);
+  float s2 = 0.f;
+  for (int c = threadIdx.x; c < d; c += 256) {
+    const float v = x[base + c] + row[c] * f * w[c];
+    x[base + c] = v;
+    row[c] = v;
+    s2 += v * v;
+    if (xcast) xcast[base + c] = from_f32<TO>(v);
+  }
+  if (!out) return;
+  const float f2 = rsqrtf(block_sum4(s2, red) / (float)d + eps_next);
+  for (int c = threadIdx.x; c < d; c += 256) out[base + c] = from_f32<TO>(row[c] * f2 * w_next[c]);
+}
+
+// x: [nt, d] float32, updated in place. delta: [planes, nt, d] float32 (planes added in order).
+// w: [d]. xcast (or null): [nt, d] receives the new rows in the engine's type. w_next / out (or
+// null): out [nt, d] = rms_norm(new x, eps_next) * w_next.
+extern "C" int ta_postnorm_add(hipStream_t stream, int out_dtype, float* x, const float* delta, int planes,
+                               long long plane, const float* w, float eps, void* xcast,
+                               const float* w_next, float eps_next, void* out, int nt, int d) {
+  TA_REQUIRE(nt >= 0 && d > 0 && d <= 32768 && planes >= 1 && planes <= TA_MAX_PLANES,
+             "ta_postnorm_add: bad sizes nt=%d d=%d planes=%d", nt, d, planes);
+  TA_REQUIRE((out == nullptr) == (w_next == nullptr), "ta_postnorm_add: w_next and out go together");
+  if (nt == 0) return 0;
+  const size_t lds = (size_t)d * sizeof(float);
+  if (out_dtype == TA_F32)
+    postnorm_add_kernel<float><<<nt, 256, lds, stream>>>(x, delta, planes, (size_t)plane, w, eps, (float*)xcast,
+                                                        w_next, eps_next, (float*)out, d);
+  else if (out_dtype == TA_BF16)
+    postnorm_add_kernel<bf16_t><<<nt, 256, lds, stream>>>(x, delta, planes, (size_t)plane, w, eps,
+                                                         (bf16_t*)xcast, w_next, eps_next, (bf16_t*)out, d);
+  else
+    return ta_fail("ta_postnorm_add: unknown dtype %d", out_dtype);
+  return ta_check_launch("ta_postnorm_add");
+}
+
+// ------------------------------------------------------------------ activations
+__device__ __forceinline__ float act_apply(int act, float z) {
+  switch (act) {
+    case 0: return 0.5f * z * (1.0f + erff(z * 0.7071067811865476f));                              // gelu
+    case 1: return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));   // gelu (tanh)
+    case 2: { const float r = fmaxf(z, 0.f); return r * r; }                                       // relu squared
+    default: return z / (1.0f + expf(-z));                                                         // silu
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void activation_kernel(const T* __restrict__ in, int in_stride,
+                                                         T* __restrict__ out, int out_stride, int n, int act,
+                                                         const float* __restrict__ side, int side_stride) {
+  const size_t t = blockIdx.y;
+  for (int c = blockIdx.x * 256 + threadIdx.x; c < n; c += gridDim.x * 256) {
+    float v = act_apply(act, to_f32(in[t * in_stride + c]));
+    if (side) v *= side[t * side_stride + c];
+    out[t * out_stride + c] = from_f32<T>(v);
+  }
+}
+
+// out[t, c] = act(in[t, c]) (* side[t, c]); rows may be strided. side: float32 or null.
+extern "C" int ta_activation(hipStream_t stream, int dtype, int act, const void* in, int in_stride, void* out,
+                             int out_stride, const float* side, int side_stride, int nt, int n) {
+  TA_REQUIRE(nt >= 0 && nt <= 65535 * 64 && n > 0 && act >= 0 && act <= 3, "ta_activation: bad sizes nt=%d n=%d act=%d", nt, n, act);
+  TA_REQUIRE(in_stride >= n && out_stride >= n && (side == nullptr || side_stride >= n), "ta_activation: strides too small");
+  for (int t0 = 0; t0 < nt; t0 += 65535) {
+    const int rows = nt - t0 < 65535 ? nt - t0 : 65535;
+    int gx = (n + 255) / 256;
+    if (gx > 64) gx = 64;
+    dim3 g(gx, rows);
+    const float* sd = side ? side + (size_t)t0 * side_stride : nullptr;
+    if (dtype == TA_F32)
+      activation_kernel<float><<<g, 256, 0, stream>>>((const float*)in + (size_t)t0 * in_stride, in_stride,
+                                                      (float*)out + (size_t)t0 * out_stride, out_stride, n, act, sd, side_stride);
+    else if (dtype == TA_BF16)
+      activation_kernel<bf16_t><<<g, 256, 0, stream>>>((const bf16_t*)in + (size_t)t0 * in_stride, in_stride,
+                                                       (bf16_t*)out + (size_t)t0 * out_stride, out_stride, n, act, sd, side_stride);
+    else
+      return ta_fail("ta_activation: unknown dtype %d", dtype);
+  }
+  return ta_check_launch("ta_activation");
+}

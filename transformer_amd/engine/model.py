@@ -226,8 +226,8 @@ class DecoderModel:
     def _stream_with(x, pending) -> torch.Tensor:
         """The residual stream with what a block has left to be added (debugging only: the
         engine itself lets the next norm do the add)."""
-        if isinstance(pending, kernels.RowScale):
-            return x.clone()                      # the block's last product has added itself
+        if isinstance(pending, (kernels.RowScale, str)):
+            return x.clone()                      # the block has added everything itself
         delta, bias = pending
         if isinstance(delta, kernels.GatedDelta):
             return delta.applied(x)

@@ -1203,3 +1203,321 @@ def gla_out(o: torch.Tensor, proj: torch.Tensor, heads: int, key_dim: int, value
                                 c_int(stride), c_int(2 * H * dk + H * dv), _ptr(weight), c_float(eps),
                                 c_int(nt), c_int(H), c_int(dv), _ptr(out)))
     return out
+
+
+# ------------------------------------------------------------------ results normed before they join the stream
+def postnorm_add(x: torch.Tensor, delta: torch.Tensor, weight: torch.Tensor, eps: float,
+                 xcast: Optional[torch.Tensor] = None, next_weight: Optional[torch.Tensor] = None,
+                 next_eps: float = 0.0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x += rms_norm(delta, eps) * weight, in float32 and in place. delta [nt, d] or
+    [planes, nt, d] float32 (planes added in order). ``xcast`` receives the new rows in its own
+    type; ``out`` = rms_norm(new x, next_eps) * next_weight (the stream's next norm, done in
+    the same pass). xcast and out share a type."""
+    _dev(x, "x", torch.float32); _dev(delta, "delta", torch.float32); _dev(weight, "weight", torch.float32)
+    nt, d = x.shape
+    planes, plane = 1, 0
+    if delta.dim() == 3 and delta.shape[1:] == x.shape:
+        planes, plane = delta.shape[0], nt * d
+    elif delta.shape != x.shape:
+        raise KernelError(f"postnorm_add: delta is {tuple(delta.shape)}, x is {tuple(x.shape)}")
+    if weight.shape != (d,):
+        raise KernelError(f"postnorm_add: weight is {tuple(weight.shape)}, expected {(d,)}")
+    code = None
+    for t, n in ((xcast, "xcast"), (out, "out")):
+        if t is not None:
+            _dev(t, n)
+            if t.shape != x.shape or (code is not None and _code(t.dtype) != code):
+                raise KernelError(f"postnorm_add: {n} is {tuple(t.shape)} {t.dtype}")
+            code = _code(t.dtype)
+    if (out is None) != (next_weight is None):
+        raise KernelError("postnorm_add: next_weight and out go together")
+    if next_weight is not None:
+        _dev(next_weight, "next_weight", torch.float32)
+        if next_weight.shape != (d,):
+            raise KernelError("postnorm_add: next_weight must have one entry per column")
+    _check(library().ta_postnorm_add(_stream(), c_int(F32 if code is None else code), _ptr(x), _ptr(delta),
+                                     c_int(planes), c_longlong(plane), _ptr(weight), c_float(eps), _ptr(xcast),
+                                     _ptr(next_weight), c_float(next_eps), _ptr(out), c_int(nt), c_int(d)))
+    return x
+
+
+_ACTIVATIONS = {"gelu": 0, "gelu_tanh": 1, "relu2": 2, "silu": 3}
+
+
+def activation(x: torch.Tensor, out: torch.Tensor, kind: str, side: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out = act(x) (* side), act "gelu" (erf), "gelu_tanh", "relu2" (relu squared) or "silu";
+    x, out [nt, n] with contiguous rows (row strides may differ); side float32 [nt, n] likewise."""
+    if kind not in _ACTIVATIONS:
+        raise KernelError(f"activation: unknown kind {kind!r}; known: {sorted(_ACTIVATIONS)}")
+    _dev(x, "x", contiguous=False); _dev(out, "out", x.dtype, contiguous=False)
+    nt, xs = _rows2d(x, "x")
+    no, os_ = _rows2d(out, "out")
+    ss = 0
+    if out.shape != x.shape:
+        raise KernelError(f"activation: x {tuple(x.shape)} / out {tuple(out.shape)}")
+    if side is not None:
+        _dev(side, "side", torch.float32, contiguous=False)
+        ns, ss = _rows2d(side, "side")
+        if side.shape != x.shape:
+            raise KernelError(f"activation: side is {tuple(side.shape)}, x {tuple(x.shape)}")
+    _check(library().ta_activation(_stream(), c_int(_code(x.dtype)), c_int(_ACTIVATIONS[kind]), _ptr(x), c_int(xs),
+                                   _ptr(out), c_int(os_), _ptr(side), c_int(ss), c_int(nt), c_int(x.shape[1])))
+    return out
+
+
+def token_shift_multi(h: torch.Tensor, out: torch.Tensor, mu: torch.Tensor, state: torch.Tensor,
+                      cu_q: torch.Tensor, slots: torch.Tensor) -> torch.Tensor:
+    """``token_shift`` with several weights at once: mu [n, d], out [n, nt, d]; out[s, t] = h[t] +
+    (h[t-1] - h[t]) * mu[s]. The state row of a sequence is read and replaced once."""
+    _dev(h, "h"); _dev(out, "out", h.dtype); _dev(mu, "mu", torch.float32); _dev(state, "state", torch.float32)
+    nt, d = h.shape
+    batch = _step_tables(cu_q, slots, nt, "token_shift_multi")
+    if mu.dim() != 2 or mu.shape[1] != d or out.shape != (mu.shape[0], nt, d) or state.dim() != 2 \
+            or state.shape[1] != d:
+        raise KernelError(f"token_shift_multi: h {tuple(h.shape)} out {tuple(out.shape)} mu {tuple(mu.shape)} "
+                          f"state {tuple(state.shape)}")
+    _check(library().ta_token_shift_multi(_stream(), c_int(_code(h.dtype)), _ptr(h), _ptr(out), _ptr(mu),
+                                          c_int(mu.shape[0]), _ptr(state), _ptr(cu_q), _ptr(slots), c_int(batch),
+                                          c_int(nt), c_int(d)))
+    return out
+
+
+def gemm_simple_batched(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[i] = a[i] @ w[i].T for 3-D views a [B, M, K], w [B, N, K], out [B, M, N] whose last
+    axis is contiguous (any batch and row strides); float32 chains as ``gemm_simple``."""
+    for t, n in ((a, "a"), (w, "w"), (out, "out")):
+        _dev(t, n, contiguous=False)
+        if t.dim() != 3 or t.stride(2) != 1:
+            raise KernelError(f"gemm_simple_batched: {n} must be 3-D with a contiguous last axis")
+    B, M, K = a.shape
+    N = w.shape[1]
+    if w.shape != (B, N, K) or out.shape != (B, M, N):
+        raise KernelError(f"gemm_simple_batched: a {tuple(a.shape)} w {tuple(w.shape)} out {tuple(out.shape)}")
+    if w.dtype != a.dtype and not (a.dtype == torch.bfloat16 and w.dtype == torch.float32):
+        raise KernelError(f"gemm_simple_batched: activations are {a.dtype}, weights {w.dtype}")
+    _check(library().ta_gemm_simple_batched(
+        _stream(), c_int(_code(a.dtype)), c_int(_code(w.dtype)), c_int(_code(out.dtype)),
+        _ptr(a), c_int(a.stride(1)), c_longlong(a.stride(0)), _ptr(w), c_int(w.stride(1)), c_longlong(w.stride(0)),
+        _ptr(None), _ptr(out), c_int(out.stride(1)), c_longlong(out.stride(0)), c_int(M), c_int(N), c_int(K), c_int(B)))
+    return out
+
+
+# ------------------------------------------------------------------ the bonus recurrence ("wkv")
+def wkv_recurrent(rkvg: torch.Tensor, low: torch.Tensor, heads: int, key_dim: int, value_dim: int, w2, w0, bonus,
+                  state: torch.Tensor, cu_q, slots, o_out: torch.Tensor, decay: torch.Tensor) -> torch.Tensor:
+    """Per head o_t = (S + diag(bonus) k_t v_t^T)^T r_t, then S <- diag(w_t) S + k_t v_t^T with
+    w_t = exp(-exp(w2 @ tanh(low_t) + w0)) per key channel. rkvg [>= 3, nt, n] planes of r, k, v
+    (n = H*dk = H*dv); low [nt, rank]; state [slots, H, dk, dv] float32; decay [nt, H*dk] float32
+    scratch that receives the decays; o_out [gla_row_parts(dk), nt, H, dv] float32 planes."""
+    _dev(rkvg, "rkvg"); _dev(low, "low", rkvg.dtype, contiguous=False)
+    H, dk, dv = heads, key_dim, value_dim
+    if rkvg.dim() != 3 or rkvg.shape[0] < 3 or dk != dv or rkvg.shape[2] != H * dk:
+        raise KernelError(f"wkv_recurrent: planes {tuple(rkvg.shape)} for {H} heads of {dk} x {dv}")
+    nt, n = rkvg.shape[1], rkvg.shape[2]
+    nl, ls = _rows2d(low, "low")
+    rank = low.shape[1]
+    batch = _step_tables(cu_q, slots, nt, "wkv_recurrent")
+    _dev(w2, "w2"); _dev(w0, "w0", torch.float32); _dev(bonus, "bonus", torch.float32)
+    _dev(state, "state", torch.float32); _dev(o_out, "o_out", torch.float32); _dev(decay, "decay", torch.float32)
+    if nl != nt or w2.shape != (n, rank) or w0.shape != (n,) or bonus.numel() != n or state.dim() != 4 \
+            or state.shape[1:] != (H, dk, dv) or o_out.shape != (gla_row_parts(dk), nt, H, dv) \
+            or decay.shape != (nt, n) or 3 * nt * n >= 2 ** 31:
+        raise KernelError(f"wkv_recurrent: shapes do not fit {H} heads of {dk}: low {tuple(low.shape)} w2 "
+                          f"{tuple(w2.shape)} state {tuple(state.shape)} o_out {tuple(o_out.shape)}")
+    _check(library().ta_wkv_recurrent(
+        _stream(), c_int(_code(rkvg.dtype)), c_int(_wcode(w2, rkvg.dtype, "wkv_recurrent")), _ptr(rkvg), c_int(n),
+        c_int(0), c_int(nt * n), c_int(2 * nt * n), _ptr(low), c_int(ls), c_int(rank), _ptr(w2), _ptr(w0),
+        _ptr(bonus), _ptr(decay), _ptr(state), _ptr(cu_q), _ptr(slots), c_int(batch), c_int(nt), c_int(H),
+        c_int(dk), c_int(dv), _ptr(o_out)))
+    return o_out
+
+
+def head_norm_gate(o: torch.Tensor, gate: torch.Tensor, heads: int, value_dim: int, weight: torch.Tensor,
+                   eps: float, out: torch.Tensor) -> torch.Tensor:
+    """out = rms_norm(o per head) * weight * silu(gate): o [parts, nt, H, dv] float32 planes that
+    add up, gate [nt, H*dv] (contiguous rows), weight [dv] for all heads or [H*dv]."""
+    _dev(o, "o", torch.float32); _dev(gate, "gate", contiguous=False); _dev(out, "out", gate.dtype)
+    _dev(weight, "weight", torch.float32)
+    nt, gs = _rows2d(gate, "gate")
+    H, dv = heads, value_dim
+    if o.dim() != 4 or o.shape[1:] != (nt, H, dv) or out.shape != (nt, H * dv) or gate.shape[1] != H * dv \
+            or weight.numel() not in (dv, H * dv):
+        raise KernelError(f"head_norm_gate: o {tuple(o.shape)} gate {tuple(gate.shape)} out {tuple(out.shape)} "
+                          f"weight {tuple(weight.shape)}")
+    _check(library().ta_gla_out_w(_stream(), c_int(_code(gate.dtype)), _ptr(o), c_int(o.shape[0]), _ptr(gate),
+                                  c_int(gs), c_longlong(0), _ptr(weight),
+                                  c_int(dv if weight.numel() == H * dv and H > 1 else 0), c_float(eps), c_int(nt),
+                                  c_int(H), c_int(dv), _ptr(out)))
+    return out
+
+
+# ------------------------------------------------------------------ attention over one latent row per token
+def latent_prepare(proj: torch.Tensor, q_rank: int, q_weight, cq, kv_offset: int, rank: int, rot: int,
+                   rot_dims: int, k_weight, eps: float, angles, dest=None, kcache=None) -> None:
+    """From rows ``proj`` [nt, >= ...]: cq [nt, q_rank] = rms_norm(first q_rank columns) *
+    q_weight (q_rank 0: no query latent); with ``dest``: the cache row of every token takes
+    rms_norm(columns kv_offset .. + rank) * k_weight and, behind it, the next ``rot`` columns
+    with the first rot_dims of them rotated in pairs (2i, 2i + 1) by ``angles`` [nt, rot_dims/2, 2]."""
+    _dev(proj, "proj", contiguous=False)
+    nt, stride = _rows2d(proj, "proj")
+    if q_rank:
+        _dev(q_weight, "q_weight", torch.float32); _dev(cq, "cq", proj.dtype)
+        if q_weight.shape != (q_rank,) or cq.shape != (nt, q_rank) or proj.shape[1] < q_rank:
+            raise KernelError(f"latent_prepare: query latent of {q_rank}: weight {tuple(q_weight.shape)} cq {tuple(cq.shape)}")
+    if dest is not None:
+        _dev(dest, "dest", torch.int32); _dev(kcache, "kcache", proj.dtype); _dev(k_weight, "k_weight", torch.float32)
+        if proj.shape[1] < kv_offset + rank + rot or k_weight.shape != (rank,) or dest.numel() != nt \
+                or kcache.dim() != 4 or tuple(kcache.shape[1:]) != (1, PAGE, rank + rot):
+            raise KernelError(f"latent_prepare: rows of {proj.shape[1]} / cache {tuple(kcache.shape)} do not fit a "
+                              f"latent of {rank} + {rot} at column {kv_offset}")
+        if rot_dims:
+            _dev(angles, "angles", torch.float32)
+            if tuple(angles.shape) != (nt, rot_dims // 2, 2):
+                raise KernelError(f"latent_prepare: angles are {tuple(angles.shape)}, expected {(nt, rot_dims // 2, 2)}")
+    _check(library().ta_latent_prepare(
+        _stream(), c_int(_code(proj.dtype)), _ptr(proj), c_int(stride), c_int(q_rank), _ptr(q_weight if q_rank else None),
+        _ptr(cq if q_rank else None), c_int(kv_offset), c_int(rank), c_int(rot), c_int(rot_dims),
+        _ptr(k_weight if dest is not None else None), c_float(eps), _ptr(angles if rot_dims else None),
+        _ptr(dest), _ptr(kcache if dest is not None else None), c_int(nt)))
+
+
+def latent_query_rot(q: torch.Tensor, heads: int, nope: int, rot: int, rot_dims: int, angles, qa: torch.Tensor,
+                     rank: int) -> torch.Tensor:
+    """qa[t, h, rank:] = the last ``rot`` coordinates of head h of q[t], the first rot_dims of
+    them rotated. q [nt, H*(nope + rot)], qa [nt, H, rank + rot]."""
+    _dev(q, "q"); _dev(qa, "qa", q.dtype)
+    nt = q.shape[0]
+    if q.shape != (nt, heads * (nope + rot)) or qa.shape != (nt, heads, rank + rot):
+        raise KernelError(f"latent_query_rot: q {tuple(q.shape)} qa {tuple(qa.shape)}")
+    if rot_dims:
+        _dev(angles, "angles", torch.float32)
+        if tuple(angles.shape) != (nt, rot_dims // 2, 2):
+            raise KernelError(f"latent_query_rot: angles are {tuple(angles.shape)}")
+    _check(library().ta_latent_query_rot(_stream(), c_int(_code(q.dtype)), _ptr(q), c_int(heads), c_int(nope),
+                                         c_int(rot), c_int(rot_dims), _ptr(angles if rot_dims else None), _ptr(qa),
+                                         c_int(rank), c_int(nt)))
+    return qa
+
+
+LATENT_MAX_RANK = 512
+
+
+def latent_attention(qa: torch.Tensor, out: torch.Tensor, kcache: torch.Tensor, block_table, cu_q, pos0,
+                     max_qlen: int, rank: int, rot: int, scale: float, window=None, gate=None) -> torch.Tensor:
+    """Causal softmax attention of wide queries qa [nt, H, rank + rot] over cached rows
+    kcache [pages, 1, PAGE, rank + rot]; out [nt, H, rank] = weighted sums of the rows' first
+    ``rank`` coordinates, times sigmoid(gate[t, h]) (gate [nt, >= H], contiguous rows)."""
+    _dev(qa, "qa"); _dev(out, "out", qa.dtype); _dev(kcache, "kcache", qa.dtype)
+    nt, H = qa.shape[0], qa.shape[1]
+    if qa.dim() != 3 or qa.shape[2] != rank + rot or out.shape != (nt, H, rank) or kcache.dim() != 4 \
+            or tuple(kcache.shape[1:]) != (1, PAGE, rank + rot):
+        raise KernelError(f"latent_attention: qa {tuple(qa.shape)} out {tuple(out.shape)} cache {tuple(kcache.shape)}")
+    _dev(block_table, "block_table", torch.int32); _dev(cu_q, "cu_q", torch.int32); _dev(pos0, "pos0", torch.int32)
+    B = pos0.numel()
+    if cu_q.numel() != B + 1 or block_table.dim() != 2 or block_table.shape[0] != B:
+        raise KernelError("latent_attention: cu_q / pos0 / block_table disagree about the batch size")
+    gs = 0
+    if gate is not None:
+        _dev(gate, "gate", qa.dtype, contiguous=False)
+        ng, gs = _rows2d(gate, "gate")
+        if ng != nt or gate.shape[1] < H:
+            raise KernelError(f"latent_attention: gate is {tuple(gate.shape)}")
+    _check(library().ta_latent_attention(
+        _stream(), c_int(_code(qa.dtype)), _ptr(qa), _ptr(out), _ptr(kcache), _ptr(block_table),
+        c_int(block_table.shape[1]), _ptr(cu_q), _ptr(pos0), c_int(B), c_int(max_qlen), c_int(H), c_int(rank),
+        c_int(rot), c_float(scale), c_int(window or 0), _ptr(gate), c_int(gs)))
+    return out
+
+
+# ------------------------------------------------------------------ routed feed-forward
+_ROUTE_MODES = {"sigmoid": 0, "softmax": 1}
+_MOE_ACTS = {None: 0, "gelu": 1, "gelu_tanh": 2, "relu2": 3, "silu": 4}
+
+
+def moe_max_rows(pairs: int, experts: int) -> int:
+    """Rows of the ordered pair list: every expert's run starts on a multiple of 16."""
+    n = int(library().ta_moe_max_rows(c_int(pairs), c_int(experts)))
+    if n < 0:
+        raise KernelError(f"moe: {pairs} pairs of {experts} experts are too many rows")
+    return n
+
+
+def moe_route(logits: torch.Tensor, experts: int, top: int, chosen: torch.Tensor, weight: torch.Tensor,
+              score: str = "sigmoid", renormalize: bool = False):
+    """chosen [nt, top] int32, weight [nt, top] float32: the ``top`` largest scores of the
+    first ``experts`` columns of logits [nt, >= experts] float32 (lowest index among equals)."""
+    _dev(logits, "logits", torch.float32, contiguous=False)
+    nt, ld = _rows2d(logits, "logits")
+    _dev(chosen, "chosen", torch.int32); _dev(weight, "weight", torch.float32)
+    if score not in _ROUTE_MODES or logits.shape[1] < experts or chosen.shape != (nt, top) or weight.shape != (nt, top):
+        raise KernelError(f"moe_route: logits {tuple(logits.shape)} chosen {tuple(chosen.shape)} score {score!r}")
+    _check(library().ta_moe_route(_stream(), _ptr(logits), c_int(ld), c_int(nt), c_int(experts), c_int(top),
+                                  c_int(_ROUTE_MODES[score]), c_int(int(renormalize)), _ptr(chosen), _ptr(weight)))
+    return chosen, weight
+
+
+def moe_plan(chosen: torch.Tensor, experts: int, row_pair: torch.Tensor, tile_expert: torch.Tensor,
+             pair_row: torch.Tensor):
+    """Orders the (token, choice) pairs by expert; see ``moe_max_rows`` for row_pair's size."""
+    _dev(chosen, "chosen", torch.int32); _dev(row_pair, "row_pair", torch.int32)
+    _dev(tile_expert, "tile_expert", torch.int32); _dev(pair_row, "pair_row", torch.int32)
+    pairs = chosen.numel()
+    rows = moe_max_rows(pairs, experts)
+    if row_pair.numel() != rows or tile_expert.numel() != rows // 16 or pair_row.numel() != pairs:
+        raise KernelError(f"moe_plan: {pairs} pairs of {experts} experts need {rows} rows")
+    _check(library().ta_moe_plan(_stream(), _ptr(chosen), c_int(pairs), c_int(experts), c_int(rows), _ptr(row_pair),
+                                 _ptr(tile_expert), _ptr(pair_row)))
+
+
+def moe_gather(h: torch.Tensor, top: int, row_pair: torch.Tensor, weight, out: torch.Tensor) -> torch.Tensor:
+    _dev(h, "h"); _dev(out, "out", h.dtype); _dev(row_pair, "row_pair", torch.int32)
+    if weight is not None:
+        _dev(weight, "weight", torch.float32)
+    if out.shape != (row_pair.numel(), h.shape[1]):
+        raise KernelError(f"moe_gather: out is {tuple(out.shape)}")
+    _check(library().ta_moe_gather(_stream(), c_int(_code(h.dtype)), _ptr(h), c_int(h.shape[1]), c_int(top),
+                                   _ptr(row_pair), _ptr(weight), _ptr(out), c_int(row_pair.numel())))
+    return out
+
+
+def moe_gemm(a: torch.Tensor, w: torch.Tensor, tile_expert: torch.Tensor, out: torch.Tensor,
+             act: Optional[str] = None) -> torch.Tensor:
+    """out[rows of tile i] = act(a[rows] @ w[tile_expert[i]].T): a [rows, K], w [E, N, K], out
+    [rows, N] in a's type or float32."""
+    _dev(a, "a"); _dev(w, "w", a.dtype); _dev(out, "out"); _dev(tile_expert, "tile_expert", torch.int32)
+    rows, K = a.shape
+    if act not in _MOE_ACTS or w.dim() != 3 or w.shape[2] != K or out.shape != (rows, w.shape[1]) \
+            or tile_expert.numel() * 16 != rows:
+        raise KernelError(f"moe_gemm: a {tuple(a.shape)} w {tuple(w.shape)} out {tuple(out.shape)} act {act!r}")
+    _check(library().ta_moe_gemm(_stream(), c_int(_code(a.dtype)), c_int(_code(out.dtype)), _ptr(a), _ptr(w),
+                                 _ptr(tile_expert), _ptr(out), c_int(rows), c_int(w.shape[1]), c_int(K),
+                                 c_int(_MOE_ACTS[act])))
+    return out
+
+
+def moe_combine(rows: torch.Tensor, top: int, pair_row: torch.Tensor, weight, shared, shared_gate,
+                delta: torch.Tensor) -> torch.Tensor:
+    """delta[t] = sum over the token's pairs of rows[pair_row] (* weight) + sigmoid(shared_gate[t,
+    0]) * shared[t]; shared [nt, d] or [planes, nt, d] float32; shared_gate float32 [nt, >= 1]."""
+    _dev(rows, "rows", torch.float32); _dev(pair_row, "pair_row", torch.int32); _dev(delta, "delta", torch.float32)
+    nt, d = delta.shape
+    if rows.shape[1] != d or pair_row.numel() != nt * top:
+        raise KernelError(f"moe_combine: rows {tuple(rows.shape)} for {nt} tokens x {top}")
+    planes, plane, gl = 1, 0, 0
+    if weight is not None:
+        _dev(weight, "weight", torch.float32)
+    if shared is not None:
+        _dev(shared, "shared", torch.float32)
+        if shared.dim() == 3 and shared.shape[1:] == delta.shape:
+            planes, plane = shared.shape[0], nt * d
+        elif shared.shape != delta.shape:
+            raise KernelError(f"moe_combine: shared is {tuple(shared.shape)}")
+    if shared_gate is not None:
+        _dev(shared_gate, "shared_gate", torch.float32, contiguous=False)
+        ng, gl = _rows2d(shared_gate, "shared_gate")
+        if ng != nt:
+            raise KernelError(f"moe_combine: shared_gate is {tuple(shared_gate.shape)}")
+    _check(library().ta_moe_combine(_stream(), _ptr(rows), c_int(d), c_int(top), _ptr(pair_row), _ptr(weight),
+                                    _ptr(shared), c_int(planes), c_longlong(plane), _ptr(shared_gate), c_int(gl),
+                                    _ptr(delta), c_int(nt)))
+    return delta

@@ -94,5 +94,92 @@ class GLU(SwiGLU):
                 self.w.get("down.bias"))
 
 
+class MLP(Part):
+    """down(act(up(h))), no gate branch (``MLPSpec``)."""
+    graph_safe = True
+
+    def __init__(self, spec, dtype, device):
+        if spec.activation not in kernels._ACTIVATIONS:
+            raise PartError(f"unknown feed-forward activation {spec.activation!r}")
+        self.spec, self.dtype = spec, dtype
+
+    def params(self):
+        s = self.spec
+        return {"up.weight": Param((s.intermediate, s.hidden), "matrix"),
+                "down.weight": Param((s.hidden, s.intermediate), "matrix")}
+
+    def run(self, h, ctx):
+        s, nt = self.spec, h.shape[0]
+        u = linear(h, self.w["up.weight"], ctx.ws.take("mlp.up", (nt, s.intermediate), self.dtype))
+        kernels.activation(u, u, s.activation)
+        return linear_delta(u, self.w["down.weight"], ctx.ws, "mlp.delta"), None
+
+
+class RoutedMLP(Part):
+    """Every token goes through the ``top`` experts with the largest router scores and,
+    optionally, a shared expert (``RoutedMLPSpec``).
+
+    One product gives the router's float32 logits (and the shared expert's gate); the chosen
+    (token, expert) pairs are ordered by expert on the GPU into a row list whose size depends
+    on the number of tokens only, so a step is the same sequence of launches whatever the
+    routing; the experts' products walk that list tile by tile, each tile with its expert's
+    matrix; the rows go back to their tokens in float32."""
+    graph_safe = True
+
+    def __init__(self, spec, dtype, device):
+        s = spec
+        if not 1 <= s.top <= s.experts or s.intermediate < 1:
+            raise PartError(f"routed feed-forward: top {s.top} of {s.experts} experts of {s.intermediate}")
+        if s.activation not in kernels._MOE_ACTS or s.activation not in kernels._ACTIVATIONS:
+            raise PartError(f"unknown expert activation {s.activation!r}")
+        if s.score not in ("sigmoid", "softmax") or s.weight_on not in ("input", "output"):
+            raise PartError(f"routed feed-forward: score {s.score!r}, weight on {s.weight_on!r}")
+        self.spec, self.dtype = s, dtype
+        self.gated_shared = s.shared_intermediate is not None and s.shared_gate
+
+    def params(self):
+        s = self.spec
+        p = {"router.weight": Param((s.experts + int(self.gated_shared), s.hidden), "matrix"),
+             "experts.up.weight": Param((s.experts * s.intermediate, s.hidden), "matrix"),
+             "experts.down.weight": Param((s.experts * s.hidden, s.intermediate), "matrix")}
+        if s.shared_intermediate is not None:
+            p["shared.up.weight"] = Param((s.shared_intermediate, s.hidden), "matrix")
+            p["shared.down.weight"] = Param((s.hidden, s.shared_intermediate), "matrix")
+        return p
+
+    def run(self, h, ctx):
+        s, nt, d = self.spec, h.shape[0], self.spec.hidden
+        E, top, ff = s.experts, s.top, s.intermediate
+        ws = ctx.ws
+        logits = linear(h, self.w["router.weight"], ws.take("moe.logits", (nt, E + int(self.gated_shared)), torch.float32))
+        chosen = ws.take("moe.chosen", (nt, top), torch.int32)
+        weight = ws.take("moe.weight", (nt, top), torch.float32)
+        kernels.moe_route(logits, E, top, chosen, weight, s.score, s.renormalize)
+        rows = kernels.moe_max_rows(nt * top, E)
+        row_pair = ws.take("moe.row_pair", (rows,), torch.int32)
+        tile_expert = ws.take("moe.tile_expert", (rows // 16,), torch.int32)
+        pair_row = ws.take("moe.pair_row", (nt * top,), torch.int32)
+        kernels.moe_plan(chosen, E, row_pair, tile_expert, pair_row)
+        on_input = s.weight_on == "input"
+        a = kernels.moe_gather(h, top, row_pair, weight if on_input else None, ws.take("moe.a", (rows, d), self.dtype))
+        up = self.w["experts.up.weight"].view(E, ff, d)
+        down = self.w["experts.down.weight"].view(E, d, ff)
+        if up.dtype != self.dtype:
+            raise PartError(f"the experts' matrices are {up.dtype}, the engine computes in {self.dtype}")
+        mid = kernels.moe_gemm(a, up, tile_expert, ws.take("moe.mid", (rows, ff), self.dtype), s.activation)
+        out = kernels.moe_gemm(mid, down, tile_expert, ws.take("moe.out", (rows, d), torch.float32))
+        shared = None
+        if s.shared_intermediate is not None:
+            u = linear(h, self.w["shared.up.weight"], ws.take("moe.shared_up", (nt, s.shared_intermediate), self.dtype))
+            kernels.activation(u, u, s.activation)
+            shared = linear_delta(u, self.w["shared.down.weight"], ws, "moe.shared")
+        delta = kernels.moe_combine(out, top, pair_row, None if on_input else weight, shared,
+                                    logits[:, E:] if self.gated_shared else None,
+                                    ws.take("moe.delta", (nt, d), torch.float32))
+        return delta, None
+
+
 register_part("swiglu", SwiGLU)
+register_part("mlp", MLP)
+register_part("routed_mlp", RoutedMLP)
 register_part("glu", GLU)

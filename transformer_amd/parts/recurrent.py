@@ -105,5 +105,59 @@ class GatedLinearAttention(Part):
         return linear_delta(g, self.w["out.weight"], ctx.ws, "gla.delta"), None
 
 
+class BonusRecurrence(Part):
+    """The matrix-state recurrence with a bonus for the current token (``BonusRecurrenceSpec``).
+
+    Its five inputs are token-shifted rows with a weight vector each; the previous token's row
+    is the first of its two pieces of state, the heads' matrices the second. The kernels are
+    those of ``GatedLinearAttention`` with the readout placed before the update (the recurrence
+    walks a sequence's tokens in order in float32; decays and state never leave float32)."""
+    graph_safe = True
+    SHIFTS = 5          # r, k, v, gate, decay: the order of the rows of ``mu``
+
+    def __init__(self, spec, dtype, device):
+        s = spec
+        if min(s.num_heads, s.head_dim, s.decay_rank) < 1:
+            raise PartError(f"bonus recurrence: heads {s.num_heads} of {s.head_dim}, decay rank {s.decay_rank}")
+        self.spec, self.dtype = s, dtype
+        self.n = s.num_heads * s.head_dim
+
+    def params(self):
+        s, n = self.spec, self.n
+        return {"mu": Param((self.SHIFTS * s.hidden,), "vector"),
+                "rkvg.weight": Param((4 * n, s.hidden), "matrix"),      # r, k, v, gate: four blocks of rows
+                "w1.weight": Param((s.decay_rank, s.hidden), "matrix"),
+                "w2.weight": Param((n, s.decay_rank), "matrix"),
+                "w0": Param((n,), "vector"),
+                "bonus": Param((s.num_heads, s.head_dim), "vector"),
+                "norm.weight": Param((n,), "vector", init="around_one"),
+                "out.weight": Param((s.hidden, n), "matrix")}
+
+    def cache_need(self):
+        s = self.spec
+        return [StateNeed((s.hidden,), torch.float32),
+                StateNeed((s.num_heads, s.head_dim, s.head_dim), torch.float32)]
+
+    def run(self, h, ctx, cache, layer, writes_cache=True):
+        s, nt, n = self.spec, h.shape[0], self.n
+        H, dk = s.num_heads, s.head_dim
+        shift_state, state = cache.layer_state(layer[0]), cache.layer_state(layer[1])
+        mixed = kernels.token_shift_multi(h, ctx.ws.take("bonus.mixed", (self.SHIFTS, nt, s.hidden), self.dtype),
+                                          self.w["mu"].view(self.SHIFTS, s.hidden), shift_state, ctx.cu_q, ctx.slots)
+        rkvg = ctx.ws.take("bonus.rkvg", (4, nt, n), self.dtype)
+        w = self.w["rkvg.weight"].view(4, n, s.hidden)
+        for i in range(4):
+            linear(mixed[i], w[i], rkvg[i])
+        low = linear(mixed[4], self.w["w1.weight"], ctx.ws.take("bonus.low", (nt, s.decay_rank), self.dtype))
+        o = kernels.wkv_recurrent(rkvg, low, H, dk, dk, self.w["w2.weight"], self.w["w0"], self.w["bonus"], state,
+                                  ctx.cu_q, ctx.slots,
+                                  ctx.ws.take("bonus.o", (kernels.gla_row_parts(dk), nt, H, dk), torch.float32),
+                                  ctx.ws.take("bonus.decay", (nt, n), torch.float32))
+        g = kernels.head_norm_gate(o, rkvg[3], H, dk, self.w["norm.weight"], float(s.eps),
+                                   ctx.ws.take("bonus.gated", (nt, n), self.dtype))
+        return linear_delta(g, self.w["out.weight"], ctx.ws, "bonus.delta"), None
+
+
 register_part("diagonal_recurrence", DiagonalRecurrence)
+register_part("bonus_recurrence", BonusRecurrence)
 register_part("gated_linear_attention", GatedLinearAttention)
