@@ -173,6 +173,51 @@ def vametar_shapes():
             "w4096": shape(4096, 32, 8, 14336, 4096, 16, 32, 128, 128, 32000)}
 
 
+def kunitar_shapes():
+    """Layer sizes that resemble real models' (random weights): Kunitar models whose layers are
+    all of one kind, the mixed order with a layer that reads its neighbour's cached rows, and the
+    Llama layer of the same width, heads and dense feed-forward. The Vametar layer with gated
+    linear attention of the same heads stands beside the recurrence (``vametar_like``)."""
+    def shape(width, heads, q_rank, kv_rank, window, ff, wkv_heads, experts, top, eff, sff, vocab):
+        dense = {"kind": "dense", "ff": ff}
+        moe = {"kind": "moe", "router": {"experts": experts, "top": top}, "expert": {"ff": eff}, "shared": {"ff": sff}}
+
+        def lat(mlp, kv_from=None):
+            m = {"heads": heads, "dim": 128, "rot_dim": 64, "vdim": 128, "q_rank": q_rank, "kv_rank": kv_rank,
+                 "scale": 192 ** -0.5, "rot": {"base": 500000.0, "dims": 64}, "mask": {"size": window}}
+            if kv_from is not None:
+                m["kv_from"] = kv_from
+            return {"type": "latent_attention", "mixer": m, "mlp": mlp}
+
+        def wkv(mlp):
+            return {"type": "wkv", "mixer": {"heads": wkv_heads, "dim": 64, "decay_rank": 64}, "mlp": mlp}
+
+        base = {"architecture": "Kunitar", "vocab": vocab, "width": width, "norm": {"eps": 1e-5},
+                "embedding": {"scale": 2.0}, "token_side": {"dim": 64}}
+        kinds = {"latent": lambda n: [lat(dense)] * n, "wkv": lambda n: [wkv(dense)] * n,
+                 "latent_moe": lambda n: [lat(moe)] * n,
+                 "mixed": lambda n: [[wkv(dense), wkv(moe), lat(moe), lat(moe, kv_from=4 * (i // 4) + 2)][i % 4]
+                                     for i in range(n)]}
+        llama = {"architectures": ["LlamaForCausalLM"], "model_type": "llama", "hidden_size": width,
+                 "num_attention_heads": heads, "num_key_value_heads": max(1, heads // 4), "head_dim": 128,
+                 "intermediate_size": ff, "vocab_size": vocab, "rope_theta": 500000.0, "rms_norm_eps": 1e-5,
+                 "tie_word_embeddings": False, "max_position_embeddings": 1 << 20, "rope_scaling": None}
+        vametar_like = {"architecture": "Vametar", "vocab": vocab, "width": width, "norm": {"eps": 1e-5},
+                        "residual_mult": 0.7, "logit_scale": 2.0,
+                        "embedding": {"bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 7}},
+                        "layers": [{"type": "gla", "mlp": {"kind": "dense", "ff": ff},
+                                    "mixer": {"heads": wkv_heads, "dim": 64, "vdim": 64, "tau": 16.0, "rank": 64}}]}
+        llama["vametar_like"] = vametar_like
+        return base, {k: f(4) for k, f in kinds.items()}, llama
+    return {"w2048": shape(2048, 16, 768, 256, 1024, 8192, 32, 32, 4, 1024, 2048, 32000),
+            "w4096": shape(4096, 32, 1536, 512, 4096, 14336, 64, 64, 6, 1408, 2816, 32000)}
+
+
+def _routed_parts(model):
+    return [b.ffn for b in model.blocks if getattr(getattr(b, "ffn", None), "spec", None) is not None
+            and getattr(b.ffn.spec, "kind", "") == "routed_mlp"]
+
+
 def generic_step_bytes(model, contexts):
     """What a single-token step reads and writes: every matrix once (of the embedding tables
     only rows), each sequence's keys and values, and its fixed-size state twice."""
@@ -195,7 +240,16 @@ def generic_step_bytes(model, contexts):
             for d in need.shape:
                 n *= d
             per_seq += 2 * n * torch.empty((), dtype=need.dtype).element_size()
-    return w + sum(contexts) * per_token + len(contexts) * per_seq
+    for f in _routed_parts(model):       # of the experts only those that the step's tokens can reach
+        sp = f.spec
+        one = 2 * sp.hidden * sp.intermediate * item
+        w -= max(0, sp.experts - len(contexts) * sp.top) * one
+    windowed = 0
+    for need in model.cache_needs:       # a window bounds what a layer reads of a sequence
+        if isinstance(need, KVNeed) and need.window is not None:
+            windowed += sum(max(0, c - need.window) for c in contexts) * need.num_kv_heads * \
+                (need.head_dim + need.value_dim) * item
+    return w + sum(contexts) * per_token - windowed + len(contexts) * per_seq
 
 
 def generic_prefill_flops(model, T):
@@ -205,19 +259,81 @@ def generic_prefill_flops(model, T):
     params = model.all_params()
     mats = sum(t.numel() for n, t in model.tensors.items()
                if params[n].role == "matrix" and n not in ("embed.weight", "head.weight", "after_embed.table"))
+    mats -= sum(t.numel() for n, t in model.tensors.items() if n.endswith(".table"))
+    for f in _routed_parts(model):       # a token goes through ``top`` of the experts
+        sp = f.spec
+        mats -= (sp.experts - sp.top) * 2 * sp.hidden * sp.intermediate
     fl = 2 * T * mats + 2 * model.spec.hidden * model.spec.vocab
     for blk in model.blocks:
         m = blk.mixer
         need = m.cache_need()
         if isinstance(need, KVNeed):
-            heads = getattr(m, "nq")
-            fl += 2 * heads * (need.head_dim + need.value_dim) * (T * (T + 1) // 2)
+            window = getattr(m.spec, "window", None)
+            pairs = T * (T + 1) // 2 if window is None or window >= T else window * (window + 1) // 2 + (T - window) * window
+            if hasattr(m, "nq"):
+                fl += 2 * m.nq * (need.head_dim + need.value_dim) * pairs
+            else:                        # one latent row per token: scores over its whole width, sums over the latent
+                fl += 2 * m.H * (need.head_dim + m.spec.kv_rank) * pairs
     return fl
 
 
 class _Vocab:
     def __init__(self, vocab):
         self.vocab = vocab
+
+
+def _design_row(model, a, dkey):
+    import torch
+    cfg = _Vocab(model.spec.vocab)
+    dt, ctx, _ = time_decode(model, cfg, a.batch, a.steps, a.warmup, 1, 512, 1024)
+    nbytes = generic_step_bytes(model, ctx)
+    pt = time_prefill(model, cfg, 3, 2, tokens=a.prefill_tokens)
+    fl = generic_prefill_flops(model, a.prefill_tokens)
+    return {"decode_tok_s": round(a.batch * a.steps / dt, 1),
+            "decode_ms_per_step": round(dt / a.steps * 1e3, 4),
+            "decode_gbs": round(nbytes / (dt / a.steps) / 1e9, 1),
+            "decode_frac_hbm": round(nbytes / (dt / a.steps) / 1e9 / HBM_GBS, 4),
+            "prefill_tok_s": round(a.prefill_tokens / pt, 1), "prefill_ms": round(pt * 1e3, 3),
+            "prefill_frac_matrix_peak": round(fl / pt / (PEAK_TFLOPS[dkey] * 1e12), 4)}
+
+
+def bench_kunitar(a):
+    """Prefill and decode throughput of Kunitar models whose layers are all of one kind, and of
+    the mixed order, beside the Llama decoder with layers of the same width, heads and dense
+    feed-forward and the Vametar decoder's gated linear attention of the recurrence's heads.
+    One JSON line of its own; the default workload is untouched."""
+    import torch
+    import transformer_amd as ta
+    dkey = "bf16" if a.dtype == "bfloat16" else "fp32"
+    layers = a.layers or 4
+    out = {"design": "kunitar", "dtype": dkey, "layers": layers, "batch": a.batch,
+           "prefill_tokens": a.prefill_tokens, "data": "synthetic", "sizes": {}}
+    for size, (base, kinds, llama) in kunitar_shapes().items():
+        if a.design_size and size not in a.design_size.split(","):
+            continue
+        llama = dict(llama)
+        vametar_like = llama.pop("vametar_like")
+        rows = {}
+        cases = [("llama", None), ("vametar_gla", None)] + list(kinds.items())
+        if a.design_case:
+            cases = [c for c in cases if c[0] in a.design_case.split(",")]
+        for name, lay in cases:
+            if name == "llama":
+                model = ta.random_model(ta.LlamaConfig.from_dict({**llama, "num_hidden_layers": layers}),
+                                        seed=0, dtype=a.dtype)
+            elif name == "vametar_gla":
+                model = ta.random_model({**vametar_like, "layers": vametar_like["layers"] * layers}, seed=0,
+                                        dtype=a.dtype, architecture="Vametar")
+            else:
+                lay = (lay * (-(-layers // len(lay))))[:layers]
+                model = ta.random_model({**base, "layers": lay}, seed=0, dtype=a.dtype, architecture="Kunitar")
+            rows[name] = _design_row(model, a, dkey)
+            del model
+            torch.cuda.empty_cache()
+            print(f"[bench] {size} {name}: {rows[name]}", file=sys.stderr, flush=True)
+        out["sizes"][size] = rows
+    print(json.dumps(out))
+    return 0
 
 
 def bench_design(a):
@@ -303,11 +419,14 @@ def main():
                     help="tokens of the prompt whose step is timed (the line's \"prefill\")")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the 2,048-token prefill (for profiling); prints its own line")
-    ap.add_argument("--design", default=None, choices=["vametar"],
+    ap.add_argument("--design", default=None, choices=["vametar", "kunitar"],
                     help="instead of the default workload: prefill and decode of this design at a few "
                          "layer sizes, beside the Llama decoder at the same sizes (a line of its own)")
     ap.add_argument("--design-size", default=None, help="with --design: only these sizes (w2048,w4096)")
+    ap.add_argument("--design-case", default=None, help="with --design kunitar: only these rows (llama,latent,...)")
     a = ap.parse_args()
+    if a.design == "kunitar" and a.gpus == 1:
+        return bench_kunitar(a)
     if a.design and a.gpus == 1:
         return bench_design(a)
     if a.gpus != 1:

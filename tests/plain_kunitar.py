@@ -153,9 +153,22 @@ def route(h, router, top):
     return order, np.take_along_axis(s, order, axis=-1)
 
 
-def moe(h, w, p, m):
+def moe(h, w, p, m, forced=None, slack=0.0):
+    """forced [T, top]: experts that another implementation chose. Where they differ from this
+    function's own choice they must be as good within ``slack`` (a close call that rounding
+    decides); the function then goes on with them, so that one close call does not change
+    everything behind it."""
     T = h.shape[0]
     chosen, weight = route(h, w[p + "router"], m["router"]["top"])
+    if forced is not None:
+        s = sigmoid(h @ w[p + "router"].T)
+        forced = np.asarray(forced, dtype=np.int64)
+        for t in range(T):
+            if set(forced[t]) != set(chosen[t]):
+                assert len(set(forced[t])) == len(forced[t]), f"token {t}: an expert chosen twice"
+                assert s[t, forced[t]].min() >= weight[t].min() - slack, \
+                    f"token {t}: experts {forced[t]} chosen, {chosen[t]} have the largest scores"
+        chosen, weight = forced, np.take_along_axis(s, forced, axis=-1)
     out = np.zeros((T, w[p + "e0.down"].shape[0]))
     for t in range(T):
         for e, g in zip(chosen[t], weight[t]):
@@ -182,9 +195,10 @@ class PlainKunitar:
             weights = read_safetensors(Path(folder) / "model.safetensors")
         self.c, self.w = config, weights
 
-    def forward(self, tokens, layers_out=None):
+    def forward(self, tokens, layers_out=None, routes=None, slack=0.03):
         """Logits [T, vocab] of a whole sequence from position 0. ``layers_out``: a list that
-        receives the residual stream after every layer."""
+        receives the residual stream after every layer. ``routes``: {layer: experts [T, top]}
+        chosen elsewhere (see ``moe``)."""
         c, w = self.c, self.w
         eps = c["norm"]["eps"]
         tokens = np.asarray(tokens, dtype=np.int64)
@@ -212,7 +226,7 @@ class PlainKunitar:
                 if mlp["kind"] == "dense":
                     f = dense_mlp(h, w, L + "mlp.")
                 elif mlp["kind"] == "moe":
-                    f = moe(h, w, L + "mlp.", mlp)
+                    f = moe(h, w, L + "mlp.", mlp, None if routes is None else routes.get(li), slack)
                 else:
                     raise ValueError(f"layer {li}: unknown feed-forward {mlp['kind']!r}")
                 x = x + rms_norm(f, w[L + "norm2b"], eps) * w[L + "ls2"]
@@ -221,3 +235,96 @@ class PlainKunitar:
             if layers_out is not None:
                 layers_out.append(x.copy())
         return rms_norm(x, w["final.norm"], eps) @ w["embed"].T
+
+
+# --------------------------------------------------------------------------
+# random models for the tests
+# --------------------------------------------------------------------------
+def tensor_shapes(c):
+    """{tensor name: shape} of a configuration, in the file's own names."""
+    d, V = c["width"], c["vocab"]
+    s = {"embed": (V, d), "final.norm": (d,)}
+    side = (c.get("token_side") or {}).get("dim")
+    if side:
+        s["side.embed"] = (V, side * len(c["layers"]))
+    for li, layer in enumerate(c["layers"]):
+        L, mx, M = f"l{li}.", layer["mixer"], f"l{li}.mix."
+        for n in ("norm1", "norm1b", "ls1"):
+            s[L + n] = (d,)
+        if layer["type"] == "latent_attention":
+            H, dn, dr, dv = mx["heads"], mx["dim"], mx["rot_dim"], mx["vdim"]
+            s[M + "dq"], s[M + "dq.norm"] = (mx["q_rank"], d), (mx["q_rank"],)
+            s[M + "uq"] = (H * (dn + dr), mx["q_rank"])
+            if mx.get("kv_from") is None:
+                s[M + "dkv"], s[M + "dkv.norm"] = (mx["kv_rank"] + dr, d), (mx["kv_rank"],)
+            s[M + "uk"], s[M + "uv"] = (H * dn, mx["kv_rank"]), (H * dv, mx["kv_rank"])
+            s[M + "g"], s[M + "o"] = (H, d), (d, H * dv)
+        else:
+            H, n, r = mx["heads"], mx["heads"] * mx["dim"], mx.get("decay_rank", 4)
+            for nme in "rkvgw":
+                s[M + "mu." + nme] = (d,)
+            for nme in "rkvg":
+                s[M + nme] = (n, d)
+            s[M + "w1"], s[M + "w2"], s[M + "w0"] = (r, d), (n, r), (n,)
+            s[M + "u"], s[M + "norm"], s[M + "o"] = (H, mx["dim"]), (n,), (d, n)
+        mlp = layer.get("mlp")
+        if mlp is not None:
+            for n in ("norm2", "norm2b", "ls2"):
+                s[L + n] = (d,)
+            F = L + "mlp."
+            if mlp["kind"] == "dense":
+                s[F + "up"], s[F + "down"] = (mlp["ff"], d), (d, mlp["ff"])
+            else:
+                for e in range(mlp["router"]["experts"]):
+                    s[f"{F}e{e}.up"], s[f"{F}e{e}.down"] = (mlp["expert"]["ff"], d), (d, mlp["expert"]["ff"])
+                s[F + "router"] = (mlp["router"]["experts"], d)
+                if mlp.get("shared") is not None:
+                    ff = mlp["shared"]["ff"]
+                    s[F + "shared.up"], s[F + "shared.down"], s[F + "shared.sg"] = (ff, d), (d, ff), (1, d)
+        if side:
+            s[L + "side.gate"], s[L + "side.proj"], s[L + "side.norm"] = (side, d), (d, side), (d,)
+    return s
+
+
+def random_weights(c, seed, edit=None):
+    """float64 weights, already rounded to bfloat16 values so that a bfloat16 file holds them
+    exactly. Matrices ~ N(0, 1/sqrt(in)); gains near 1; shift weights in (0, 1); decays between
+    0.4 and 0.95 a step; router rows large enough that the chosen experts are no close call."""
+    rng = np.random.default_rng(seed)
+    w = {}
+    for name, shape in tensor_shapes(c).items():
+        last = name.rsplit(".", 1)[-1]
+        if last in ("norm1", "norm2", "norm1b", "norm2b", "norm"):
+            a = 1.0 + 0.2 * rng.standard_normal(shape)
+        elif last in ("ls1", "ls2"):
+            a = 0.7 + 0.2 * rng.standard_normal(shape)
+        elif ".mu." in name:
+            a = rng.uniform(0.1, 0.9, shape)
+        elif last == "w0":
+            a = rng.uniform(-3.0, 0.0, shape)
+        elif last == "u":
+            a = 0.5 * rng.standard_normal(shape)
+        elif last == "router":
+            a = 4.0 * rng.standard_normal(shape) / np.sqrt(shape[-1])
+        elif name in ("embed", "side.embed"):
+            a = rng.standard_normal(shape)
+        else:
+            a = rng.standard_normal(shape) / np.sqrt(shape[-1])
+        w[name] = round_bf16(a)
+    if edit is not None:
+        edit(w)
+        for n in w:
+            w[n] = round_bf16(w[n].reshape(-1)).reshape(w[n].shape)
+    return w
+
+
+def make_model_folder(folder, c, seed, storage="BF16", edit=None):
+    folder = Path(folder)
+    folder.mkdir(parents=True, exist_ok=True)
+    w = random_weights(c, seed, edit)
+    write_safetensors(folder / "model.safetensors", w, dtype=storage)
+    cfg = json.loads(json.dumps(c))
+    for layer in cfg["layers"]:                       # the file says it: a tensor's shape
+        layer["mixer"].pop("decay_rank", None)
+    (folder / "config.json").write_text(json.dumps(cfg, indent=1))
+    return w

@@ -100,6 +100,7 @@ class StepContext:
         self.ws: Optional[Workspace] = None
         self.shared = {}     # what parts compute once per step and share (cleared by every run)
         self.timers = None   # parts.base.PartTimers while the model collects times per kind of part
+        self.dump = None     # dump(name, tensor) of the run in progress while the model's ``dump`` is set
         self.real_batch = 0  # sequences of the caller; the rest of ``batch`` only fills a launch shape
         self.real_want = 0
 

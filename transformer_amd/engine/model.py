@@ -193,6 +193,8 @@ class DecoderModel:
         pending = (None, None)
         for i, run in enumerate(s.schedule):
             block = self.blocks[run.block]
+            # a part may hand intermediates of its own to the dump: ``ctx.dump(name, tensor)``
+            ctx.dump = None if self.dump is None else (lambda n, t, i=i: self.dump(f"run.{i}.{n}", t))
             kw = {}
             if getattr(block, "folds_norms", False) and i + 1 < len(s.schedule):
                 kw["after"] = self.blocks[s.schedule[i + 1].block]    # it may prepare that block's norm

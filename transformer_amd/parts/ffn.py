@@ -155,6 +155,8 @@ class RoutedMLP(Part):
         chosen = ws.take("moe.chosen", (nt, top), torch.int32)
         weight = ws.take("moe.weight", (nt, top), torch.float32)
         kernels.moe_route(logits, E, top, chosen, weight, s.score, s.renormalize)
+        if getattr(ctx, "dump", None) is not None:
+            ctx.dump("experts", chosen)
         rows = kernels.moe_max_rows(nt * top, E)
         row_pair = ws.take("moe.row_pair", (rows,), torch.int32)
         tile_expert = ws.take("moe.tile_expert", (rows // 16,), torch.int32)
