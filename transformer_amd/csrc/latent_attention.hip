@@ -38,7 +38,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void latent_prepare_kernel(
     const T* __restrict__ proj, int stride, int q_rank, const float* __restrict__ qw, T* __restrict__ cq,
     int kvoff, int rank, int rot, int rot_dims, const float* __restrict__ kw, float eps,
-    const float* __restrict__ angles, const int* __restrict__ dest, T* __restrict__ kcache) {
+    const float* __restrict__ angles, const int* __restrict__ dest, T* __restrict__ kcache, int dc) {
   __shared__ float red[4];
   const size_t t = blockIdx.x;
   const T* row = proj + t * stride;
@@ -60,8 +60,9 @@ __global__ __launch_bounds__(256) void latent_prepare_kernel(
     ss += v * v;
   }
   const float f = rsqrtf(la_block_sum(ss, red) / (float)rank + eps);
-  T* out = kcache + (size_t)dest[t] * (rank + rot);
+  T* out = kcache + (size_t)dest[t] * dc;
   for (int c = threadIdx.x; c < rank; c += 256) out[c] = from_f32<T>(to_f32(kv[c]) * f * kw[c]);
+  for (int c = rank + rot + threadIdx.x; c < dc; c += 256) out[c] = from_f32<T>(0.f);
   const float* ang = angles + t * (size_t)rot_dims;          // (cos, sin) pairs: rot_dims floats a token
   for (int i = threadIdx.x; i < rot / 2 + (rot & 1); i += 256) {
     const float u = to_f32(kv[rank + 2 * i]);
@@ -80,22 +81,24 @@ __global__ __launch_bounds__(256) void latent_prepare_kernel(
 
 // proj: [nt, stride] rows: the query latent (q_rank) first, the key/value latent (rank) and the
 // shared key part (rot) from column kvoff. cq: [nt, q_rank]. dest null: the step's rows store
-// nothing (the layer reads rows that another layer stored). kcache: [pages, 1, PAGE, rank + rot].
+// nothing (the layer reads rows that another layer stored). kcache: [pages, 1, PAGE, dc], dc >=
+// rank + rot; the rest of a row is zeroed.
 extern "C" int ta_latent_prepare(hipStream_t stream, int dtype, const void* proj, int stride, int q_rank,
                                  const float* qw, void* cq, int kvoff, int rank, int rot, int rot_dims,
                                  const float* kw, float eps, const float* angles, const int* dest,
-                                 void* kcache, int nt) {
+                                 void* kcache, int dc, int nt) {
   TA_REQUIRE(nt >= 0 && q_rank >= 0 && rank >= 1 && rot >= 0 && rot_dims >= 0 && rot_dims <= rot && rot_dims % 2 == 0,
              "ta_latent_prepare: bad sizes nt=%d q_rank=%d rank=%d rot=%d dims=%d", nt, q_rank, rank, rot, rot_dims);
   TA_REQUIRE(q_rank > 0 || dest != nullptr, "ta_latent_prepare: nothing to do");
+  TA_REQUIRE(dest == nullptr || dc >= rank + rot, "ta_latent_prepare: cache rows of %d for %d + %d", dc, rank, rot);
   TA_REQUIRE(dest == nullptr || rot_dims == 0 || angles != nullptr, "ta_latent_prepare: angles are required");
   if (nt == 0) return 0;
   if (dtype == TA_F32)
     latent_prepare_kernel<float><<<nt, 256, 0, stream>>>((const float*)proj, stride, q_rank, qw, (float*)cq, kvoff, rank,
-                                                        rot, rot_dims, kw, eps, angles, dest, (float*)kcache);
+                                                        rot, rot_dims, kw, eps, angles, dest, (float*)kcache, dc);
   else if (dtype == TA_BF16)
     latent_prepare_kernel<bf16_t><<<nt, 256, 0, stream>>>((const bf16_t*)proj, stride, q_rank, qw, (bf16_t*)cq, kvoff,
-                                                         rank, rot, rot_dims, kw, eps, angles, dest, (bf16_t*)kcache);
+                                                         rank, rot, rot_dims, kw, eps, angles, dest, (bf16_t*)kcache, dc);
   else
     return ta_fail("ta_latent_prepare: unknown dtype %d", dtype);
   return ta_check_launch("ta_latent_prepare");
@@ -105,14 +108,18 @@ extern "C" int ta_latent_prepare(hipStream_t stream, int dtype, const void* proj
 template <typename T>
 __global__ __launch_bounds__(256) void latent_query_rot_kernel(const T* __restrict__ q, int H, int dn, int rot,
                                                                int rot_dims, const float* __restrict__ angles,
-                                                               T* __restrict__ qa, int rank) {
+                                                               T* __restrict__ qa, int rank, int dc) {
   const size_t t = blockIdx.x;
+  for (int idx = threadIdx.x; idx < H * (dc - rank - rot); idx += 256) {      // the rows' padding
+    const int h = idx / (dc - rank - rot), i = idx % (dc - rank - rot);
+    qa[(t * H + h) * (size_t)dc + rank + rot + i] = from_f32<T>(0.f);
+  }
   const float* ang = angles + t * (size_t)rot_dims;
   const int pairs = (rot + 1) / 2;
   for (int idx = threadIdx.x; idx < H * pairs; idx += 256) {
     const int h = idx / pairs, i = idx % pairs;
     const T* src = q + (t * H + h) * (size_t)(dn + rot) + dn;
-    T* dst = qa + (t * H + h) * (size_t)(rank + rot) + rank;
+    T* dst = qa + (t * H + h) * (size_t)dc + rank;
     const float u = to_f32(src[2 * i]);
     if (2 * i + 1 >= rot) { dst[2 * i] = from_f32<T>(u); continue; }
     const float v = to_f32(src[2 * i + 1]);
@@ -127,17 +134,18 @@ __global__ __launch_bounds__(256) void latent_query_rot_kernel(const T* __restri
   }
 }
 
-// q: [nt, H, dn + rot] (each head: unrotated part, then the part to rotate); qa: [nt, H, rank + rot],
-// whose last rot coordinates per head are written.
+// q: [nt, H, dn + rot] (each head: unrotated part, then the part to rotate); qa: [nt, H, dc], dc >=
+// rank + rot, whose coordinates from ``rank`` on are written (the rotated part, then zeros).
 extern "C" int ta_latent_query_rot(hipStream_t stream, int dtype, const void* q, int H, int dn, int rot,
-                                   int rot_dims, const float* angles, void* qa, int rank, int nt) {
+                                   int rot_dims, const float* angles, void* qa, int rank, int dc, int nt) {
   TA_REQUIRE(nt >= 0 && H >= 1 && dn >= 0 && rot >= 0 && rank >= 1 && rot_dims >= 0 && rot_dims <= rot && rot_dims % 2 == 0,
              "ta_latent_query_rot: bad sizes");
-  if (nt == 0 || rot == 0) return 0;
+  TA_REQUIRE(dc >= rank + rot, "ta_latent_query_rot: rows of %d for %d + %d", dc, rank, rot);
+  if (nt == 0 || dc == rank) return 0;
   if (dtype == TA_F32)
-    latent_query_rot_kernel<float><<<nt, 256, 0, stream>>>((const float*)q, H, dn, rot, rot_dims, angles, (float*)qa, rank);
+    latent_query_rot_kernel<float><<<nt, 256, 0, stream>>>((const float*)q, H, dn, rot, rot_dims, angles, (float*)qa, rank, dc);
   else if (dtype == TA_BF16)
-    latent_query_rot_kernel<bf16_t><<<nt, 256, 0, stream>>>((const bf16_t*)q, H, dn, rot, rot_dims, angles, (bf16_t*)qa, rank);
+    latent_query_rot_kernel<bf16_t><<<nt, 256, 0, stream>>>((const bf16_t*)q, H, dn, rot, rot_dims, angles, (bf16_t*)qa, rank, dc);
   else
     return ta_fail("ta_latent_query_rot: unknown dtype %d", dtype);
   return ta_check_launch("ta_latent_query_rot");
@@ -166,7 +174,7 @@ __global__ __launch_bounds__(256) void latent_attention_kernel(
     const T* __restrict__ qa, T* __restrict__ out, const T* __restrict__ kcache,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ cu_q,
     const int* __restrict__ pos0, int H, int rank, int rot, float scale, int window,
-    const T* __restrict__ gate, int gate_stride) {
+    const T* __restrict__ gate, int gate_stride, int dc) {
   extern __shared__ float smem[];
   const int D = rank + rot, DP = D + 1;
   const int b = blockIdx.y;
@@ -186,7 +194,7 @@ __global__ __launch_bounds__(256) void latent_attention_kernel(
 
   for (int i = threadIdx.x; i < LA_ROWS * D; i += 256) {
     const int r = i / D, d = i - r * D, rr = row0 + r;
-    Qs[i] = rr < nrows ? to_f32(qa[((size_t)(q0 + rr / H) * H + rr % H) * D + d]) : 0.f;
+    Qs[i] = rr < nrows ? to_f32(qa[((size_t)(q0 + rr / H) * H + rr % H) * dc + d]) : 0.f;
   }
   const int qi_min = row0 / H;
   const int last_row = (row0 + LA_ROWS - 1 < nrows - 1) ? row0 + LA_ROWS - 1 : nrows - 1;
@@ -210,11 +218,11 @@ __global__ __launch_bounds__(256) void latent_attention_kernel(
   for (int c = tile_start / LA_CHUNK; c * LA_CHUNK < tile_end; ++c) {
     const int key0 = c * LA_CHUNK;
     const size_t page = (size_t)table[key0 / TA_PAGE];
-    const size_t base = (page * TA_PAGE + key0 % TA_PAGE) * (size_t)D;
+    const size_t base = (page * TA_PAGE + key0 % TA_PAGE) * (size_t)dc;
     __syncthreads();                         // the chunk before has been read
     for (int i = threadIdx.x; i < LA_CHUNK * D; i += 256) {
       const int k = i / D, d = i - k * D;
-      Ks[k * DP + d] = (key0 + k < tile_end) ? to_f32(kcache[base + i]) : 0.f;
+      Ks[k * DP + d] = (key0 + k < tile_end) ? to_f32(kcache[base + (size_t)k * dc + d]) : 0.f;
     }
     __syncthreads();
     float s0 = 0.f, s1 = 0.f;
@@ -275,7 +283,7 @@ template <typename T, int NACC>
 static int latent_attention_run(hipStream_t stream, dim3 g, size_t lds, const void* qa, void* out,
                                 const void* kcache, const int* block_table, int max_blocks, const int* cu_q,
                                 const int* pos0, int H, int rank, int rot, float scale, int window,
-                                const void* gate, int gate_stride) {
+                                const void* gate, int gate_stride, int dc) {
   auto kern = latent_attention_kernel<T, NACC>;
   if (lds > 64 * 1024) {
     const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -283,22 +291,313 @@ static int latent_attention_run(hipStream_t stream, dim3 g, size_t lds, const vo
     if (e != hipSuccess) return ta_fail("ta_latent_attention: %zu bytes of LDS refused (%s)", lds, hipGetErrorString(e));
   }
   kern<<<g, 256, lds, stream>>>((const T*)qa, (T*)out, (const T*)kcache, block_table, max_blocks, cu_q, pos0, H,
-                                rank, rot, scale, window, (const T*)gate, gate_stride);
+                                rank, rot, scale, window, (const T*)gate, gate_stride, dc);
   return 0;
 }
 
-// qa: [nt, H, rank + rot] wide queries. out: [nt, H, rank]. kcache: one layer,
-// [pages][1][TA_PAGE][rank + rot]. gate (or null): pre-activation of a sigmoid gate per
+// ------------------------------------------------------------------ the same on the matrix cores (bfloat16)
+// A wave owns RT tiles of 16 rows and a share of their keys; a workgroup is four such waves that
+// share nothing (no barrier between them). Keys come in chunks of 32 aligned to absolute
+// positions: the wave copies a chunk's rows into its own piece of LDS, forms S^T = K Q^T on
+// v_mfma_f32_16x16x32_bf16 (a lane then holds 4 keys x 2 tiles of ONE row: the softmax stays in
+// the lane but for two shuffles), and O^T += C^T P^T with the latent's coordinates gathered
+// from the same LDS rows. Scores, maxima, sums and weights are float32; a weight enters the
+// second product as THREE bfloat16 pieces (p = p0 + p1 + p2 exactly: 3 x 8 bits of mantissa), so
+// the product sees all of its 24 bits and only the cached rows are bfloat16.
+// With `splits` > 1 a tile's chunks are dealt to that many waves, which leave (sums, maximum,
+// sum of weights) in `partial` for `latent_merge_kernel`: steps of single tokens have few rows
+// and long key ranges.
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 la_bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float la_floatx4;
+union LaFrag {
+  la_bf16x8 v;
+  uint4 q;
+  uint32_t w[4];
+  uint16_t s[8];
+};
+
+template <int KS, int CT, int RT>
+__global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
+    const bf16_t* __restrict__ qa, bf16_t* __restrict__ out, const bf16_t* __restrict__ kcache,
+    const int* __restrict__ block_table, int max_blocks, const int* __restrict__ cu_q,
+    const int* __restrict__ pos0, int H, int rank, int dc, float scale_log2, int window,
+    const bf16_t* __restrict__ gate, int gate_stride, int splits, int tiles_max, float* __restrict__ partial) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char la_lds[];
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+  const int c = lane % 16, g = lane / 16;
+  const int RS = dc + 8;                                  // elements between rows of the LDS copy
+  bf16_t* Ks = reinterpret_cast<bf16_t*>(la_lds) + (size_t)wave * 32 * RS;
+  const int b = blockIdx.y, split = blockIdx.z;
+  const int q0 = cu_q[b], qlen = cu_q[b + 1] - q0;
+  const int nrows = qlen * H;
+  const int tile = blockIdx.x * 4 + wave;
+  const int row0 = tile * 16 * RT;
+  if (row0 >= nrows) return;                              // a wave leaves alone: nothing below waits for others
+  const int p0 = pos0[b];
+  int my_start[RT], my_end[RT];
+  bool ok[RT];
+  LaFrag qf[RT][KS];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const int row = row0 + 16 * rt + c;
+    ok[rt] = row < nrows;
+    const int qi = ok[rt] ? row / H : 0;
+    my_end[rt] = p0 + qi + 1;
+    my_start[rt] = window > 0 ? (my_end[rt] - window > 0 ? my_end[rt] - window : 0) : 0;
+    const bf16_t* qrow = qa + ((size_t)q0 * H + (ok[rt] ? row : 0)) * dc;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int d = 32 * ks + 8 * g;
+      qf[rt][ks].q = (ok[rt] && d < dc) ? *reinterpret_cast<const uint4*>(qrow + d) : uint4{0, 0, 0, 0};
+    }
+  }
+  const int last_row = (row0 + 16 * RT - 1 < nrows - 1) ? row0 + 16 * RT - 1 : nrows - 1;
+  const int tile_end = p0 + last_row / H + 1;
+  int tile_start = 0;
+  if (window > 0) {
+    tile_start = p0 + row0 / H + 1 - window;
+    if (tile_start < 0) tile_start = 0;
+  }
+  const int c0 = tile_start / 32, c1 = (tile_end + 31) / 32;
+  const int n = c1 - c0;
+  const int ca = c0 + (int)((long long)n * split / splits), cb = c0 + (int)((long long)n * (split + 1) / splits);
+  la_floatx4 O[RT][CT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) O[rt][ct] = la_floatx4{0.f, 0.f, 0.f, 0.f};
+  float m[RT], l[RT];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) { m[rt] = -INFINITY; l[rt] = 0.f; }
+  const int* table = block_table + (size_t)b * max_blocks;
+  const int pieces = dc / 8;                              // 16-byte pieces of a row
+  for (int ch = ca; ch < cb; ++ch) {
+    const int key0 = ch * 32;
+    const size_t page = (size_t)table[key0 / TA_PAGE];
+    const bf16_t* src = kcache + (page * TA_PAGE + key0 % TA_PAGE) * (size_t)dc;
+    __builtin_amdgcn_wave_barrier();                      // the chunk before has been read
+    for (int idx = lane; idx < 32 * pieces; idx += 64) {
+      const int k = idx / pieces, pc = idx - k * pieces;
+      const uint4 v = (key0 + k < tile_end) ? *reinterpret_cast<const uint4*>(src + (size_t)k * dc + pc * 8)
+                                            : uint4{0, 0, 0, 0};        // keys not written yet read as zero
+      *reinterpret_cast<uint4*>(Ks + k * RS + pc * 8) = v;
+    }
+    __builtin_amdgcn_wave_barrier();
+    // ---- scores: register j of tile t of a lane is key 16 t + 4 g + j for the lane's row c
+    la_floatx4 S[RT][2];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int t = 0; t < 2; ++t) S[rt][t] = la_floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int d = 32 * ks + 8 * g;
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        LaFrag kf;
+        kf.q = d < dc ? *reinterpret_cast<const uint4*>(Ks + (16 * t + c) * RS + d) : uint4{0, 0, 0, 0};
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+          S[rt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qf[rt][ks].v, S[rt][t], 0, 0, 0);
+      }
+    }
+    // ---- softmax of the lane's rows over the chunk, in the log2 domain
+    LaFrag pf[RT][3];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      float sv[8];
+      float mx = -INFINITY;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int key = key0 + 16 * (e / 4) + 4 * g + (e % 4);
+        const bool vis = ok[rt] && key >= my_start[rt] && key < my_end[rt];
+        sv[e] = vis ? S[rt][e / 4][e % 4] * scale_log2 : -INFINITY;
+        mx = fmaxf(mx, sv[e]);
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, TA_WAVE));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, TA_WAVE));
+      const float m_new = fmaxf(m[rt], mx);
+      const float m_use = m_new == -INFINITY ? 0.f : m_new;
+      const float alpha = exp2f(m[rt] - m_use);          // m = -inf gives 0
+      float rs = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float p = exp2f(sv[e] - m_use);             // -inf gives 0
+        rs += p;
+        const float h0 = to_f32(from_f32<bf16_t>(p));
+        const float r1 = p - h0;
+        const float h1 = to_f32(from_f32<bf16_t>(r1));
+        const float r2 = r1 - h1;
+        pf[rt][0].s[e] = f32_to_bf16_bits(p);
+        pf[rt][1].s[e] = f32_to_bf16_bits(r1);
+        pf[rt][2].s[e] = f32_to_bf16_bits(r2);
+      }
+      rs += __shfl_xor(rs, 16, TA_WAVE);
+      rs += __shfl_xor(rs, 32, TA_WAVE);
+      l[rt] = l[rt] * alpha + rs;
+      m[rt] = m_new;
+      if (alpha != 1.f) {
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) O[rt][ct][j] *= alpha;
+      }
+    }
+    // ---- weighted sums: the lane brings coordinate 16 ct + c of its 8 keys
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+      const int coord = 16 * ct + c;
+      if (16 * ct >= rank) break;
+      LaFrag vf;
+      const uint16_t* col = reinterpret_cast<const uint16_t*>(Ks) + (coord < rank ? coord : 0);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const uint16_t v = col[(16 * (e / 4) + 4 * g + (e % 4)) * RS];
+        vf.s[e] = coord < rank ? v : (uint16_t)0;
+      }
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int sp = 0; sp < 3; ++sp)
+          O[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[rt][sp].v, O[rt][ct], 0, 0, 0);
+    }
+  }
+  // ---- results: register j of tile ct is coordinate 16 ct + 4 g + j of the lane's row c
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    if (!ok[rt]) continue;
+    const int row = row0 + 16 * rt + c;
+    if (splits > 1) {
+      float* dst = partial + ((((size_t)b * tiles_max + tile) * splits + split) * (16 * RT) + 16 * rt + c) * (rank + 2);
+#pragma unroll
+      for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int coord = 16 * ct + 4 * g + j;
+          if (coord < rank) dst[coord] = O[rt][ct][j];
+        }
+      if (g == 0) { dst[rank] = m[rt]; dst[rank + 1] = l[rt]; }
+      continue;
+    }
+    float f = l[rt] > 0.f ? 1.0f / l[rt] : 0.f;
+    if (gate) {
+      const float gv = to_f32(gate[(size_t)(q0 + row / H) * gate_stride + row % H]);
+      f *= 1.0f / (1.0f + expf(-gv));
+    }
+    bf16_t* o = out + ((size_t)q0 * H + row) * rank;
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int coord = 16 * ct + 4 * g + j;
+        if (coord < rank) o[coord] = from_f32<bf16_t>(O[rt][ct][j] * f);
+      }
+  }
+}
+
+// One wave per row: the shares of a row's keys are put together.
+__global__ __launch_bounds__(64) void latent_merge_kernel(const float* __restrict__ partial, bf16_t* __restrict__ out,
+                                                          const int* __restrict__ cu_q, int H, int rank, int splits,
+                                                          int tiles_max, int rows_per_tile,
+                                                          const bf16_t* __restrict__ gate, int gate_stride) {
+  const int b = blockIdx.y, row = blockIdx.x;
+  const int q0 = cu_q[b], qlen = cu_q[b + 1] - q0;
+  if (row >= qlen * H) return;
+  const int tile = row / rows_per_tile, rl = row % rows_per_tile;
+  const float* base = partial + (((size_t)b * tiles_max + tile) * splits * rows_per_tile + rl) * (rank + 2);
+  const size_t step = (size_t)rows_per_tile * (rank + 2);
+  float M = -INFINITY;
+  for (int s = 0; s < splits; ++s) M = fmaxf(M, base[s * step + rank]);
+  float L = 0.f;
+  for (int s = 0; s < splits; ++s) {
+    const float ms = base[s * step + rank];
+    if (ms != -INFINITY) L += exp2f(ms - M) * base[s * step + rank + 1];
+  }
+  float f = L > 0.f ? 1.0f / L : 0.f;
+  if (gate) {
+    const float gv = to_f32(gate[(size_t)(q0 + row / H) * gate_stride + row % H]);
+    f *= 1.0f / (1.0f + expf(-gv));
+  }
+  bf16_t* o = out + ((size_t)q0 * H + row) * rank;
+  for (int cdx = threadIdx.x; cdx < rank; cdx += 64) {
+    float acc = 0.f;
+    for (int s = 0; s < splits; ++s) {
+      const float ms = base[s * step + rank];
+      if (ms != -INFINITY) acc += exp2f(ms - M) * base[s * step + cdx];
+    }
+    o[cdx] = from_f32<bf16_t>(acc * f);
+  }
+}
+
+template <int KS, int CT, int RT>
+static int latent_mfma_run(hipStream_t stream, dim3 g, size_t lds, const void* qa, void* out, const void* kcache,
+                           const int* block_table, int max_blocks, const int* cu_q, const int* pos0, int H,
+                           int rank, int dc, float scale_log2, int window, const void* gate, int gate_stride,
+                           int splits, int tiles_max, float* partial) {
+  auto kern = latent_attention_mfma_kernel<KS, CT, RT>;
+  if (lds > 64 * 1024) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return ta_fail("ta_latent_attention: %zu bytes of LDS refused (%s)", lds, hipGetErrorString(e));
+  }
+  kern<<<g, 256, lds, stream>>>((const bf16_t*)qa, (bf16_t*)out, (const bf16_t*)kcache, block_table, max_blocks,
+                                cu_q, pos0, H, rank, dc, scale_log2, window, (const bf16_t*)gate, gate_stride, splits,
+                                tiles_max, partial);
+  return 0;
+}
+
+// Rows per tile that the matrix-core kernel gives a wave for this geometry (0: it does not take
+// it), and the float32 values of scratch that `splits` shares of the keys need.
+extern "C" int ta_latent_mfma_rows(int rank, int dc, int max_qlen, int H) {
+  if (dc % 8 || rank < 1 || rank > 512 || dc > 576 || dc < rank) return 0;
+  if (dc <= 192 && rank <= 128) return (long long)max_qlen * H >= 64 ? 32 : 16;
+  return 16;
+}
+extern "C" long long ta_latent_mfma_scratch(int batch, int max_qlen, int H, int rank, int dc, int splits) {
+  const int rows = ta_latent_mfma_rows(rank, dc, max_qlen, H);
+  if (rows == 0 || splits <= 1) return 0;
+  const long long tiles = ((long long)max_qlen * H + rows - 1) / rows;
+  return (long long)batch * tiles * splits * rows * (rank + 2);
+}
+
+// qa: [nt, H, dc] wide queries (dc >= rank + rot, the rest zero). out: [nt, H, rank]. kcache: one
+// layer, [pages][1][TA_PAGE][dc]. gate (or null): pre-activation of a sigmoid gate per
 // (token, head), element h of a row of gate_stride elements. window <= 0: all earlier keys.
+// bfloat16 with rows of whole 16-byte pieces runs on the matrix cores; `splits` > 1 deals a
+// row's keys to that many waves (scratch: ta_latent_mfma_scratch floats). float32, and rows
+// that are no multiple of 8 wide, run on the vector ALU (splits is ignored).
 extern "C" int ta_latent_attention(hipStream_t stream, int dtype, const void* qa, void* out, const void* kcache,
                                    const int* block_table, int max_blocks, const int* cu_q, const int* pos0,
-                                   int batch, int max_qlen, int H, int rank, int rot, float scale, int window,
-                                   const void* gate, int gate_stride) {
+                                   int batch, int max_qlen, int H, int rank, int rot, int dc, float scale, int window,
+                                   const void* gate, int gate_stride, int splits, float* scratch) {
   TA_REQUIRE(batch >= 0 && batch <= 65535 && max_qlen >= 0 && H >= 1, "ta_latent_attention: bad batch=%d max_qlen=%d heads=%d", batch, max_qlen, H);
   TA_REQUIRE(rank >= 1 && rank <= 512 && rot >= 0 && rot <= 512, "ta_latent_attention: latent of %d / rotated part of %d outside [1, 512] / [0, 512]", rank, rot);
+  TA_REQUIRE(dc >= rank + rot, "ta_latent_attention: rows of %d for %d + %d", dc, rank, rot);
   TA_REQUIRE(max_blocks > 0, "ta_latent_attention: empty block table");
   TA_REQUIRE(gate == nullptr || gate_stride >= H, "ta_latent_attention: gate rows too short");
   if (batch == 0 || max_qlen == 0) return 0;
+  const int rows = dtype == TA_BF16 ? ta_latent_mfma_rows(rank, dc, max_qlen, H) : 0;
+  if (rows > 0) {
+    TA_REQUIRE(splits >= 1 && splits <= 65535 && (splits == 1 || scratch != nullptr), "ta_latent_attention: %d shares without scratch", splits);
+    const long long tiles = ((long long)max_qlen * H + rows - 1) / rows;
+    TA_REQUIRE(tiles <= 2147483647ll, "ta_latent_attention: too many rows");
+    dim3 g((unsigned)((tiles + 3) / 4), batch, splits);
+    const size_t lds = (size_t)4 * 32 * (dc + 8) * sizeof(bf16_t);
+    const float sl2 = scale * 1.4426950408889634f;
+    int rc;
+#define LA_MFMA(KS, CT, RT) latent_mfma_run<KS, CT, RT>(stream, g, lds, qa, out, kcache, block_table, max_blocks, cu_q, pos0, H, rank, dc, sl2, window, gate, gate_stride, splits, (int)tiles, scratch)
+    if (dc <= 192 && rank <= 128) rc = rows == 32 ? LA_MFMA(6, 8, 2) : LA_MFMA(6, 8, 1);
+    else if (dc <= 320 && rank <= 256) rc = LA_MFMA(10, 16, 1);
+    else rc = LA_MFMA(18, 32, 1);
+#undef LA_MFMA
+    if (rc) return rc;
+    if (splits > 1) {
+      dim3 gm((unsigned)(max_qlen * H), batch);
+      latent_merge_kernel<<<gm, 64, 0, stream>>>(scratch, (bf16_t*)out, cu_q, H, rank, splits, (int)tiles, rows,
+                                                 (const bf16_t*)gate, gate_stride);
+    }
+    return ta_check_launch("ta_latent_attention");
+  }
   const long long tiles = ((long long)max_qlen * H + LA_ROWS - 1) / LA_ROWS;
   TA_REQUIRE(tiles <= 2147483647ll, "ta_latent_attention: too many rows");
   dim3 g((unsigned)tiles, batch);
@@ -307,9 +606,9 @@ extern "C" int ta_latent_attention(hipStream_t stream, int dtype, const void* qa
   TA_REQUIRE(lds <= 160 * 1024, "ta_latent_attention: rows of %d do not fit the LDS", D);
   int rc;
 #define LA_RUN(T)                                                                                              \
-  (rank <= 128 ? latent_attention_run<T, 8>(stream, g, lds, qa, out, kcache, block_table, max_blocks, cu_q, pos0, H, rank, rot, scale, window, gate, gate_stride)   \
-   : rank <= 256 ? latent_attention_run<T, 16>(stream, g, lds, qa, out, kcache, block_table, max_blocks, cu_q, pos0, H, rank, rot, scale, window, gate, gate_stride) \
-                 : latent_attention_run<T, 32>(stream, g, lds, qa, out, kcache, block_table, max_blocks, cu_q, pos0, H, rank, rot, scale, window, gate, gate_stride))
+  (rank <= 128 ? latent_attention_run<T, 8>(stream, g, lds, qa, out, kcache, block_table, max_blocks, cu_q, pos0, H, rank, rot, scale, window, gate, gate_stride, dc)   \
+   : rank <= 256 ? latent_attention_run<T, 16>(stream, g, lds, qa, out, kcache, block_table, max_blocks, cu_q, pos0, H, rank, rot, scale, window, gate, gate_stride, dc) \
+                 : latent_attention_run<T, 32>(stream, g, lds, qa, out, kcache, block_table, max_blocks, cu_q, pos0, H, rank, rot, scale, window, gate, gate_stride, dc))
   if (dtype == TA_F32) rc = LA_RUN(float);
   else if (dtype == TA_BF16) rc = LA_RUN(bf16_t);
   else return ta_fail("ta_latent_attention: unknown dtype %d", dtype);

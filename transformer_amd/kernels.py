@@ -1367,7 +1367,7 @@ def latent_prepare(proj: torch.Tensor, q_rank: int, q_weight, cq, kv_offset: int
     if dest is not None:
         _dev(dest, "dest", torch.int32); _dev(kcache, "kcache", proj.dtype); _dev(k_weight, "k_weight", torch.float32)
         if proj.shape[1] < kv_offset + rank + rot or k_weight.shape != (rank,) or dest.numel() != nt \
-                or kcache.dim() != 4 or tuple(kcache.shape[1:]) != (1, PAGE, rank + rot):
+                or kcache.dim() != 4 or tuple(kcache.shape[1:3]) != (1, PAGE) or kcache.shape[3] < rank + rot:
             raise KernelError(f"latent_prepare: rows of {proj.shape[1]} / cache {tuple(kcache.shape)} do not fit a "
                               f"latent of {rank} + {rot} at column {kv_offset}")
         if rot_dims:
@@ -1378,16 +1378,17 @@ def latent_prepare(proj: torch.Tensor, q_rank: int, q_weight, cq, kv_offset: int
         _stream(), c_int(_code(proj.dtype)), _ptr(proj), c_int(stride), c_int(q_rank), _ptr(q_weight if q_rank else None),
         _ptr(cq if q_rank else None), c_int(kv_offset), c_int(rank), c_int(rot), c_int(rot_dims),
         _ptr(k_weight if dest is not None else None), c_float(eps), _ptr(angles if rot_dims else None),
-        _ptr(dest), _ptr(kcache if dest is not None else None), c_int(nt)))
+        _ptr(dest), _ptr(kcache if dest is not None else None),
+        c_int(kcache.shape[3] if dest is not None else rank + rot), c_int(nt)))
 
 
 def latent_query_rot(q: torch.Tensor, heads: int, nope: int, rot: int, rot_dims: int, angles, qa: torch.Tensor,
                      rank: int) -> torch.Tensor:
     """qa[t, h, rank:] = the last ``rot`` coordinates of head h of q[t], the first rot_dims of
-    them rotated. q [nt, H*(nope + rot)], qa [nt, H, rank + rot]."""
+    them rotated, then zeros up to the rows' width. q [nt, H*(nope + rot)], qa [nt, H, >= rank + rot]."""
     _dev(q, "q"); _dev(qa, "qa", q.dtype)
     nt = q.shape[0]
-    if q.shape != (nt, heads * (nope + rot)) or qa.shape != (nt, heads, rank + rot):
+    if q.shape != (nt, heads * (nope + rot)) or qa.dim() != 3 or qa.shape[:2] != (nt, heads) or qa.shape[2] < rank + rot:
         raise KernelError(f"latent_query_rot: q {tuple(q.shape)} qa {tuple(qa.shape)}")
     if rot_dims:
         _dev(angles, "angles", torch.float32)
@@ -1395,22 +1396,46 @@ def latent_query_rot(q: torch.Tensor, heads: int, nope: int, rot: int, rot_dims:
             raise KernelError(f"latent_query_rot: angles are {tuple(angles.shape)}")
     _check(library().ta_latent_query_rot(_stream(), c_int(_code(q.dtype)), _ptr(q), c_int(heads), c_int(nope),
                                          c_int(rot), c_int(rot_dims), _ptr(angles if rot_dims else None), _ptr(qa),
-                                         c_int(rank), c_int(nt)))
+                                         c_int(rank), c_int(qa.shape[2]), c_int(nt)))
     return qa
 
 
 LATENT_MAX_RANK = 512
 
 
+def latent_row_width(rank: int, rot: int, dtype: torch.dtype) -> int:
+    """Numbers a cached row (and a wide query) holds: rank + rot, rounded up to whole 16-byte
+    pieces for bfloat16 so that the matrix-core kernel takes them (the rest is zero)."""
+    return -(-(rank + rot) // 8) * 8 if dtype == torch.bfloat16 else rank + rot
+
+
+def latent_key_shares(batch: int, max_qlen: int, heads: int, rank: int, width: int, max_kv_len: int,
+                      window: Optional[int]) -> int:
+    """Waves that share a row's keys in ``latent_attention`` on the matrix cores: one when the
+    step's rows alone give the CUs enough waves, else enough to reach about two waves per SIMD
+    while a share keeps at least two chunks of 32 keys. A function of the step's shape only."""
+    rows = int(library().ta_latent_mfma_rows(c_int(rank), c_int(width), c_int(max_qlen), c_int(heads)))
+    if rows == 0:
+        return 1
+    waves = batch * -(-max_qlen * heads // rows)
+    keys = max_kv_len if not window else min(max_kv_len, window + max_qlen)
+    chunks = keys // 32 + 2
+    return max(1, min(chunks // 2, 2048 // max(waves, 1)))
+
+
 def latent_attention(qa: torch.Tensor, out: torch.Tensor, kcache: torch.Tensor, block_table, cu_q, pos0,
-                     max_qlen: int, rank: int, rot: int, scale: float, window=None, gate=None) -> torch.Tensor:
-    """Causal softmax attention of wide queries qa [nt, H, rank + rot] over cached rows
-    kcache [pages, 1, PAGE, rank + rot]; out [nt, H, rank] = weighted sums of the rows' first
-    ``rank`` coordinates, times sigmoid(gate[t, h]) (gate [nt, >= H], contiguous rows)."""
+                     max_qlen: int, rank: int, rot: int, scale: float, window=None, gate=None,
+                     shares: int = 1) -> torch.Tensor:
+    """Causal softmax attention of wide queries qa [nt, H, width] over cached rows kcache
+    [pages, 1, PAGE, width] (width >= rank + rot, the rest zero); out [nt, H, rank] = weighted
+    sums of the rows' first ``rank`` coordinates, times sigmoid(gate[t, h]) (gate [nt, >= H],
+    contiguous rows). bfloat16 rows of whole 16-byte pieces run on the matrix cores, where
+    ``shares`` waves divide a row's keys (``latent_key_shares``); all else on the vector ALU."""
     _dev(qa, "qa"); _dev(out, "out", qa.dtype); _dev(kcache, "kcache", qa.dtype)
     nt, H = qa.shape[0], qa.shape[1]
-    if qa.dim() != 3 or qa.shape[2] != rank + rot or out.shape != (nt, H, rank) or kcache.dim() != 4 \
-            or tuple(kcache.shape[1:]) != (1, PAGE, rank + rot):
+    width = qa.shape[2] if qa.dim() == 3 else -1
+    if qa.dim() != 3 or width < rank + rot or out.shape != (nt, H, rank) or kcache.dim() != 4 \
+            or tuple(kcache.shape[1:]) != (1, PAGE, width):
         raise KernelError(f"latent_attention: qa {tuple(qa.shape)} out {tuple(out.shape)} cache {tuple(kcache.shape)}")
     _dev(block_table, "block_table", torch.int32); _dev(cu_q, "cu_q", torch.int32); _dev(pos0, "pos0", torch.int32)
     B = pos0.numel()
@@ -1422,10 +1447,20 @@ def latent_attention(qa: torch.Tensor, out: torch.Tensor, kcache: torch.Tensor, 
         ng, gs = _rows2d(gate, "gate")
         if ng != nt or gate.shape[1] < H:
             raise KernelError(f"latent_attention: gate is {tuple(gate.shape)}")
+    scratch = None
+    if shares > 1:
+        need = library().ta_latent_mfma_scratch
+        need.restype = c_longlong
+        floats = need(c_int(B), c_int(max_qlen), c_int(H), c_int(rank), c_int(width), c_int(shares))
+        if floats > 0 and qa.dtype == torch.bfloat16:
+            scratch = _scratch_floats(qa.device, floats)
+        else:
+            shares = 1
     _check(library().ta_latent_attention(
         _stream(), c_int(_code(qa.dtype)), _ptr(qa), _ptr(out), _ptr(kcache), _ptr(block_table),
         c_int(block_table.shape[1]), _ptr(cu_q), _ptr(pos0), c_int(B), c_int(max_qlen), c_int(H), c_int(rank),
-        c_int(rot), c_float(scale), c_int(window or 0), _ptr(gate), c_int(gs)))
+        c_int(rot), c_int(width), c_float(scale), c_int(window or 0), _ptr(gate), c_int(gs), c_int(shares),
+        _ptr(scratch)))
     return out
 
 

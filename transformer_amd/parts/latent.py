@@ -47,6 +47,7 @@ class LatentAttention(Part):
         self.kv_off = s.q_rank
         self.gate_off = s.q_rank + (s.kv_rank + s.rope_dim if s.own_kv else 0)
         self.width = self.gate_off + (self.H if s.gated else 0)
+        self.row = kernels.latent_row_width(s.kv_rank, s.rope_dim, dtype)      # a cached row, a wide query
         self.rotary = None
         if s.rot_dims:
             self.rotary = build_part(PositionSpec(head_dim=s.rot_dims, theta=s.rot_base, style="interleaved"),
@@ -66,7 +67,7 @@ class LatentAttention(Part):
 
     def cache_need(self):
         s = self.spec
-        return KVNeed(1, s.kv_rank + s.rope_dim, s.cache_window, 0)
+        return KVNeed(1, self.row, s.cache_window, 0)
 
     def bind(self, tensors):
         super().bind(tensors)
@@ -98,16 +99,17 @@ class LatentAttention(Part):
                                self.w.get("kv_norm.weight"), float(s.eps), angles,
                                meta.dest if s.own_kv else None, kc if s.own_kv else None)
         q = linear(cq, self.w["uq.weight"], ctx.ws.take("latent.q", (nt, H * (self.dn + dr)), self.dtype))
-        qa = ctx.ws.take("latent.qa", (nt, H, r + dr), self.dtype)
+        qa = ctx.ws.take("latent.qa", (nt, H, self.row), self.dtype)
         kernels.latent_query_rot(q, H, self.dn, dr, s.rot_dims, angles, qa, r)
         if self.dn:
             self._per_head(q.view(nt, H, self.dn + dr)[:, :, :self.dn], self.uk_t, qa[:, :, :r])
         else:
             qa[:, :, :r].zero_()
         ol = ctx.ws.take("latent.ol", (nt, H, r), self.dtype)
+        shares = kernels.latent_key_shares(ctx.batch, ctx.max_qlen, H, r, self.row, ctx.max_kv_len, s.window)
         kernels.latent_attention(qa, ol, kc, meta.block_table, ctx.cu_q, ctx.pos0, ctx.max_qlen, r, dr,
                                  float(s.scale), s.window,
-                                 gate=proj[:, self.gate_off:] if s.gated else None)
+                                 gate=proj[:, self.gate_off:] if s.gated else None, shares=shares)
         o = ctx.ws.take("latent.o", (nt, H, self.dv), self.dtype)
         self._per_head(ol, self.uv, o)
         return linear_delta(o.view(nt, H * self.dv), self.w["out.weight"], ctx.ws, "latent.delta"), None
