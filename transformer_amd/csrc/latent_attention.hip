@@ -317,7 +317,7 @@ union LaFrag {
 };
 
 template <int KS, int CT, int RT>
-__global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
+__global__ __launch_bounds__(256, (KS <= 6 ? 2 : 1)) void latent_attention_mfma_kernel(
     const bf16_t* __restrict__ qa, bf16_t* __restrict__ out, const bf16_t* __restrict__ kcache,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ cu_q,
     const int* __restrict__ pos0, int H, int rank, int dc, float scale_log2, int window,
@@ -371,16 +371,46 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
   for (int rt = 0; rt < RT; ++rt) { m[rt] = -INFINITY; l[rt] = 0.f; }
   const int* table = block_table + (size_t)b * max_blocks;
   const int pieces = dc / 8;                              // 16-byte pieces of a row
-  for (int ch = ca; ch < cb; ++ch) {
+  // A chunk is 32 * pieces pieces, NL = 2 KS of them a lane at most. With PRE they are asked for
+  // one chunk ahead and wait in registers while the chunk before is multiplied.
+  constexpr int NL = 2 * KS;
+  constexpr bool PRE = KS <= 10;
+  uint4 pre[PRE ? NL : 1];
+  auto fetch = [&](int ch, uint4* buf, int i0, int i1) {
     const int key0 = ch * 32;
     const size_t page = (size_t)table[key0 / TA_PAGE];
     const bf16_t* src = kcache + (page * TA_PAGE + key0 % TA_PAGE) * (size_t)dc;
-    __builtin_amdgcn_wave_barrier();                      // the chunk before has been read
-    for (int idx = lane; idx < 32 * pieces; idx += 64) {
+#pragma unroll
+    for (int i = i0; i < i1; ++i) {
+      const int idx = lane + 64 * i;
       const int k = idx / pieces, pc = idx - k * pieces;
-      const uint4 v = (key0 + k < tile_end) ? *reinterpret_cast<const uint4*>(src + (size_t)k * dc + pc * 8)
-                                            : uint4{0, 0, 0, 0};        // keys not written yet read as zero
-      *reinterpret_cast<uint4*>(Ks + k * RS + pc * 8) = v;
+      const bool live = idx < 32 * pieces && key0 + k < tile_end;       // keys not written yet read as zero
+      const uint4 v = *reinterpret_cast<const uint4*>(live ? src + (size_t)k * dc + pc * 8 : kcache);
+      buf[i - i0] = live ? v : uint4{0, 0, 0, 0};
+    }
+  };
+  auto stash = [&](const uint4* buf, int i0, int i1) {
+#pragma unroll
+    for (int i = i0; i < i1; ++i) {
+      const int idx = lane + 64 * i;
+      const int k = idx / pieces, pc = idx - k * pieces;
+      if (idx < 32 * pieces) *reinterpret_cast<uint4*>(Ks + k * RS + pc * 8) = buf[i - i0];
+    }
+  };
+  if (PRE && ca < cb) fetch(ca, pre, 0, NL);
+  for (int ch = ca; ch < cb; ++ch) {
+    const int key0 = ch * 32;
+    __builtin_amdgcn_wave_barrier();                      // the chunk before has been read
+    if (PRE) {
+      stash(pre, 0, NL);
+      if (ch + 1 < cb) fetch(ch + 1, pre, 0, NL);
+    } else {
+#pragma unroll
+      for (int i0 = 0; i0 < NL; i0 += 12) {
+        uint4 buf[12];
+        fetch(ch, buf, i0, i0 + 12 < NL ? i0 + 12 : NL);
+        stash(buf, i0, i0 + 12 < NL ? i0 + 12 : NL);
+      }
     }
     __builtin_amdgcn_wave_barrier();
     // ---- scores: register j of tile t of a lane is key 16 t + 4 g + j for the lane's row c
@@ -418,16 +448,14 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
       mx = fmaxf(mx, __shfl_xor(mx, 32, TA_WAVE));
       const float m_new = fmaxf(m[rt], mx);
       const float m_use = m_new == -INFINITY ? 0.f : m_new;
-      const float alpha = exp2f(m[rt] - m_use);          // m = -inf gives 0
+      const float alpha = __builtin_amdgcn_exp2f(m[rt] - m_use);       // m = -inf gives 0
       float rs = 0.f;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
-        const float p = exp2f(sv[e] - m_use);             // -inf gives 0
+        const float p = __builtin_amdgcn_exp2f(sv[e] - m_use);          // -inf gives 0
         rs += p;
-        const float h0 = to_f32(from_f32<bf16_t>(p));
-        const float r1 = p - h0;
-        const float h1 = to_f32(from_f32<bf16_t>(r1));
-        const float r2 = r1 - h1;
+        const float r1 = p - to_f32(from_f32<bf16_t>(p));
+        const float r2 = r1 - to_f32(from_f32<bf16_t>(r1));
         pf[rt][0].s[e] = f32_to_bf16_bits(p);
         pf[rt][1].s[e] = f32_to_bf16_bits(r1);
         pf[rt][2].s[e] = f32_to_bf16_bits(r2);
@@ -436,33 +464,44 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
       rs += __shfl_xor(rs, 32, TA_WAVE);
       l[rt] = l[rt] * alpha + rs;
       m[rt] = m_new;
-      if (alpha != 1.f) {
+      if (__any(alpha != 1.f)) {
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct)
 #pragma unroll
           for (int j = 0; j < 4; ++j) O[rt][ct][j] *= alpha;
       }
     }
-    // ---- weighted sums: the lane brings coordinate 16 ct + c of its 8 keys
+    // ---- weighted sums. A lane reads 4 neighbouring coordinates (8 bytes) of each of its 8
+    // keys and feeds four products from them: in product q of a block of 64 coordinates row i
+    // of the first operand stands for coordinate 4 i + q, so register j of O[4 qb + q] is
+    // coordinate 64 qb + 16 g + 4 j + q of the lane's row c.
 #pragma unroll
-    for (int ct = 0; ct < CT; ++ct) {
-      const int coord = 16 * ct + c;
-      if (16 * ct >= rank) break;
-      LaFrag vf;
-      const uint16_t* col = reinterpret_cast<const uint16_t*>(Ks) + (coord < rank ? coord : 0);
+    for (int qb = 0; qb < CT / 4; ++qb) {
+      if (64 * qb >= rank) break;
+      int col = 64 * qb + 4 * c;
+      if (col > RS - 4) col = RS - 4;                     // past the row: coordinates nobody stores
+      uint2 wv[8];
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const uint16_t v = col[(16 * (e / 4) + 4 * g + (e % 4)) * RS];
-        vf.s[e] = coord < rank ? v : (uint16_t)0;
+      for (int e = 0; e < 8; ++e)
+        wv[e] = *reinterpret_cast<const uint2*>(Ks + (16 * (e / 4) + 4 * g + (e % 4)) * RS + col);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        LaFrag vf;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const uint32_t lo = q < 2 ? wv[2 * i].x : wv[2 * i].y, hi = q < 2 ? wv[2 * i + 1].x : wv[2 * i + 1].y;
+          vf.w[i] = __builtin_amdgcn_perm(hi, lo, (q & 1) ? 0x07060302u : 0x05040100u);
+        }
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+          for (int sp = 0; sp < 3; ++sp)
+            O[rt][4 * qb + q] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[rt][sp].v, O[rt][4 * qb + q], 0, 0, 0);
       }
-#pragma unroll
-      for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-        for (int sp = 0; sp < 3; ++sp)
-          O[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[rt][sp].v, O[rt][ct], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
-  // ---- results: register j of tile ct is coordinate 16 ct + 4 g + j of the lane's row c
+  // ---- results: register j of O[4 qb + q] is coordinate 64 qb + 16 g + 4 j + q of the lane's row c
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
     if (!ok[rt]) continue;
@@ -473,7 +512,7 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
       for (int ct = 0; ct < CT; ++ct)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          const int coord = 16 * ct + 4 * g + j;
+          const int coord = 64 * (ct / 4) + 16 * g + 4 * j + (ct % 4);
           if (coord < rank) dst[coord] = O[rt][ct][j];
         }
       if (g == 0) { dst[rank] = m[rt]; dst[rank + 1] = l[rt]; }
@@ -489,7 +528,7 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
     for (int ct = 0; ct < CT; ++ct)
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const int coord = 16 * ct + 4 * g + j;
+        const int coord = 64 * (ct / 4) + 16 * g + 4 * j + (ct % 4);
         if (coord < rank) o[coord] = from_f32<bf16_t>(O[rt][ct][j] * f);
       }
   }
@@ -506,13 +545,19 @@ __global__ __launch_bounds__(64) void latent_merge_kernel(const float* __restric
   const int tile = row / rows_per_tile, rl = row % rows_per_tile;
   const float* base = partial + (((size_t)b * tiles_max + tile) * splits * rows_per_tile + rl) * (rank + 2);
   const size_t step = (size_t)rows_per_tile * (rank + 2);
+  extern __shared__ float wts[];          // [splits] weight of every share
   float M = -INFINITY;
-  for (int s = 0; s < splits; ++s) M = fmaxf(M, base[s * step + rank]);
+  for (int s = threadIdx.x; s < splits; s += 64) M = fmaxf(M, base[s * step + rank]);
+  M = wave_max(M);
   float L = 0.f;
-  for (int s = 0; s < splits; ++s) {
+  for (int s = threadIdx.x; s < splits; s += 64) {
     const float ms = base[s * step + rank];
-    if (ms != -INFINITY) L += exp2f(ms - M) * base[s * step + rank + 1];
+    const float w = ms != -INFINITY ? exp2f(ms - M) : 0.f;
+    wts[s] = w;
+    L += w * base[s * step + rank + 1];
   }
+  L = wave_sum(L);
+  __syncthreads();
   float f = L > 0.f ? 1.0f / L : 0.f;
   if (gate) {
     const float gv = to_f32(gate[(size_t)(q0 + row / H) * gate_stride + row % H]);
@@ -521,10 +566,8 @@ __global__ __launch_bounds__(64) void latent_merge_kernel(const float* __restric
   bf16_t* o = out + ((size_t)q0 * H + row) * rank;
   for (int cdx = threadIdx.x; cdx < rank; cdx += 64) {
     float acc = 0.f;
-    for (int s = 0; s < splits; ++s) {
-      const float ms = base[s * step + rank];
-      if (ms != -INFINITY) acc += exp2f(ms - M) * base[s * step + cdx];
-    }
+#pragma unroll 8
+    for (int s = 0; s < splits; ++s) acc = fmaf(wts[s], base[s * step + cdx], acc);     // shares in order
     o[cdx] = from_f32<bf16_t>(acc * f);
   }
 }
@@ -593,7 +636,7 @@ extern "C" int ta_latent_attention(hipStream_t stream, int dtype, const void* qa
     if (rc) return rc;
     if (splits > 1) {
       dim3 gm((unsigned)(max_qlen * H), batch);
-      latent_merge_kernel<<<gm, 64, 0, stream>>>(scratch, (bf16_t*)out, cu_q, H, rank, splits, (int)tiles, rows,
+      latent_merge_kernel<<<gm, 64, (size_t)splits * sizeof(float), stream>>>(scratch, (bf16_t*)out, cu_q, H, rank, splits, (int)tiles, rows,
                                                  (const bf16_t*)gate, gate_stride);
     }
     return ta_check_launch("ta_latent_attention");

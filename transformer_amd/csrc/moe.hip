@@ -10,7 +10,8 @@
 //                 acts on the expert's input
 //   moe_gemm    : C[rows of a tile] = A[rows] * W[expert of the tile]^T for all tiles, with an
 //                 optional activation; float32 chains on the vector ALU, or the matrix cores
-//                 (v_mfma_f32_16x16x32_bf16) for bfloat16
+//                 (v_mfma_f32_16x16x32_bf16) for bfloat16, where neighbouring tiles of one
+//                 expert share every load of its matrix
 //   moe_combine : delta[t] = sum of the token's pairs' rows (times the weight when it acts on
 //                 the output) + sigmoid(shared gate) * the shared expert's rows
 //
@@ -236,21 +237,111 @@ union MoeFrag {
   moe_u32x4 q;
 };
 
-// Matrix cores: a workgroup of 4 waves owns a tile of 16 rows; a wave 64 columns (four 16 x 16
-// tiles) and walks K in steps of 32: a lane holds 8 consecutive k of row (lane % 16) of its
-// operand. K % 8 == 0; the last step's missing k are zero.
+// Matrix cores: a workgroup of 4 waves owns four neighbouring tiles of 16 rows, a wave 64
+// columns of them (four 16 x 16 tiles). Neighbouring tiles of one expert form a run; a wave
+// walks K once per run, in steps of 32 (a lane holds 8 consecutive k of row lane % 16 of its
+// operand), and every piece of the expert's matrix that it loads serves all tiles of the run:
+// a prompt's rows, of which an expert gets many, read the matrix a quarter as often; a step of
+// few tokens has runs of one tile and reads every chosen expert's matrix once. The operands of
+// the next step are asked for before the products of this one. K % 8 == 0; the last step's
+// missing k are zero.
+template <typename TC, int RUN>
+__device__ __forceinline__ void moe_run(const bf16_t* __restrict__ A, const bf16_t* __restrict__ We,
+                                        TC* __restrict__ C, size_t r0, int n0, int N, int K, int act, int lane) {
+  const int r = lane % 16, kb = lane / 16;
+  const bf16_t* arow[RUN];
+#pragma unroll
+  for (int u = 0; u < RUN; ++u) arow[u] = A + (r0 + 16 * u + r) * K + kb * 8;
+  const bf16_t* wrow[4];
+  bool wok[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    const int n = n0 + 16 * t + r;
+    wok[t] = n < N;
+    wrow[t] = We + (size_t)(wok[t] ? n : 0) * K + kb * 8;
+  }
+  moe_floatx4 acc[RUN][4];
+#pragma unroll
+  for (int u = 0; u < RUN; ++u)
+#pragma unroll
+    for (int t = 0; t < 4; ++t) acc[u][t] = moe_floatx4{0.f, 0.f, 0.f, 0.f};
+  const moe_u32x4 zero = {0, 0, 0, 0};
+  MoeFrag af[RUN], wf[4], an[RUN], wn[4];
+  auto load = [&](MoeFrag* a, MoeFrag* w, int k0) {
+    const bool kok = k0 + kb * 8 < K;
+#pragma unroll
+    for (int u = 0; u < RUN; ++u) a[u].q = kok ? *reinterpret_cast<const moe_u32x4*>(arow[u] + k0) : zero;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+      w[t].q = (kok && wok[t]) ? __builtin_nontemporal_load(reinterpret_cast<const moe_u32x4*>(wrow[t] + k0)) : zero;
+  };
+  load(af, wf, 0);
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    if (k0 + 32 < K) load(an, wn, k0 + 32);
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int u = 0; u < RUN; ++u)
+        // register j of a lane: W row 4 * (lane / 16) + j of the tile, activation row lane % 16
+        acc[u][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[t].v, af[u].v, acc[u][t], 0, 0, 0);
+#pragma unroll
+    for (int u = 0; u < RUN; ++u) af[u] = an[u];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) wf[t] = wn[t];
+  }
+#pragma unroll
+  for (int u = 0; u < RUN; ++u)
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int n = n0 + 16 * t + 4 * kb + j;
+        if (n < N) C[(r0 + 16 * u + r) * N + n] = from_f32<TC>(moe_act(act, acc[u][t][j]));
+      }
+}
+
 template <typename TC>
 __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W,
-                                                            const int* __restrict__ tile_expert,
+                                                            const int* __restrict__ tile_expert, int tiles,
                                                             TC* __restrict__ C, int N, int K, int act) {
-  const int e = tile_expert[blockIdx.y];
-  if (e < 0) return;
-  const size_t r0 = (size_t)blockIdx.y * MOE_TILE;
   const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   const int n0 = (blockIdx.x * 4 + wave) * 64;
   if (n0 >= N) return;
-  const bf16_t* We = W + (size_t)e * N * K;
+  int t = blockIdx.y * 4;
+  const int t_end = t + 4 < tiles ? t + 4 : tiles;
+  while (t < t_end) {
+    const int e = tile_expert[t];
+    if (e < 0) return;                                  // tiles past the last expert's rows
+    int run = 1;
+    while (t + run < t_end && tile_expert[t + run] == e) ++run;
+    const bf16_t* We = W + (size_t)e * N * K;
+    const size_t r0 = (size_t)t * MOE_TILE;
+    if (run == 4) moe_run<TC, 4>(A, We, C, r0, n0, N, K, act, lane);
+    else if (run == 3) moe_run<TC, 3>(A, We, C, r0, n0, N, K, act, lane);
+    else if (run == 2) moe_run<TC, 2>(A, We, C, r0, n0, N, K, act, lane);
+    else moe_run<TC, 1>(A, We, C, r0, n0, N, K, act, lane);
+    t += run;
+  }
+}
+
+// Few tiles (a step of few tokens): a workgroup owns ONE tile of 16 rows and 64 columns and its
+// four waves divide K, so that four times as many loads of the expert's matrix are on their way;
+// the partial tiles are added in wave order through LDS.
+template <typename TC>
+__global__ __launch_bounds__(256) void moe_gemm_mfma_splitk_kernel(const bf16_t* __restrict__ A,
+                                                                   const bf16_t* __restrict__ W,
+                                                                   const int* __restrict__ tile_expert,
+                                                                   TC* __restrict__ C, int N, int K, int act) {
+  __shared__ float red[4][16][65];
+  const int e = tile_expert[blockIdx.y];
+  if (e < 0) return;                                    // the whole workgroup: tiles past the last expert's rows
+  const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
   const int r = lane % 16, kb = lane / 16;
+  const int n0 = blockIdx.x * 64;
+  const size_t r0 = (size_t)blockIdx.y * MOE_TILE;
+  const bf16_t* We = W + (size_t)e * N * K;
+  const int steps = (K + 31) / 32;
+  const int kbeg = 32 * (steps * wave / 4), kend = 32 * (steps * (wave + 1) / 4);
   const bf16_t* arow = A + (r0 + r) * K + kb * 8;
   const bf16_t* wrow[4];
   bool wok[4];
@@ -264,25 +355,35 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16_t* __rest
 #pragma unroll
   for (int t = 0; t < 4; ++t) acc[t] = moe_floatx4{0.f, 0.f, 0.f, 0.f};
   const moe_u32x4 zero = {0, 0, 0, 0};
-  for (int k0 = 0; k0 < K; k0 += 32) {
-    const bool kok = k0 + kb * 8 < K;
-    MoeFrag af;
-    af.q = kok ? *reinterpret_cast<const moe_u32x4*>(arow + k0) : zero;
+  constexpr int DEPTH = 4;                              // steps of 32 k asked for together
+  for (int k0 = kbeg; k0 < kend; k0 += 32 * DEPTH) {
+    MoeFrag af[DEPTH], wf[DEPTH][4];
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      MoeFrag wf;
-      wf.q = (kok && wok[t]) ? *reinterpret_cast<const moe_u32x4*>(wrow[t] + k0) : zero;
-      // register j of a lane: W row 4 * (lane / 16) + j of the tile, activation row lane % 16
-      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf.v, af.v, acc[t], 0, 0, 0);
+    for (int u = 0; u < DEPTH; ++u) {
+      const int k = k0 + 32 * u;
+      const bool kok = k < kend && k + kb * 8 < K;
+      af[u].q = kok ? *reinterpret_cast<const moe_u32x4*>(arow + k) : zero;
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+        wf[u][t].q = (kok && wok[t]) ? __builtin_nontemporal_load(reinterpret_cast<const moe_u32x4*>(wrow[t] + k)) : zero;
     }
+#pragma unroll
+    for (int u = 0; u < DEPTH; ++u)
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[u][t].v, af[u].v, acc[t], 0, 0, 0);
   }
 #pragma unroll
   for (int t = 0; t < 4; ++t)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int n = n0 + 16 * t + 4 * kb + j;
-      if (n < N) C[(r0 + r) * N + n] = from_f32<TC>(moe_act(act, acc[t][j]));
-    }
+    for (int j = 0; j < 4; ++j) red[wave][r][16 * t + 4 * kb + j] = acc[t][j];
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int idx = threadIdx.x + 256 * i, row = idx / 64, col = idx % 64;
+    const float v = (red[0][row][col] + red[1][row][col]) + (red[2][row][col] + red[3][row][col]);
+    if (n0 + col < N) C[(r0 + row) * N + n0 + col] = from_f32<TC>(moe_act(act, v));
+  }
 }
 
 // A: [max_rows, K] ordered rows; W: [E, N, K]; C: [max_rows, N], float32 or the type of A;
@@ -295,11 +396,20 @@ extern "C" int ta_moe_gemm(hipStream_t stream, int dtype, int out_dtype, const v
   if (max_rows == 0) return 0;
   const int tiles = max_rows / MOE_TILE;
   if (dtype == TA_BF16 && K % 8 == 0) {
-    dim3 g((N + 255) / 256, tiles);
+    if (out_dtype != TA_BF16 && out_dtype != TA_F32) return ta_fail("ta_moe_gemm: unknown output type %d", out_dtype);
+    if ((long long)tiles * ((N + 255) / 256) < 1024) {   // too few workgroups to fill the CUs: the waves divide K
+      dim3 gk((N + 63) / 64, tiles);
+      if (out_dtype == TA_BF16)
+        moe_gemm_mfma_splitk_kernel<bf16_t><<<gk, 256, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, tile_expert, (bf16_t*)C, N, K, act);
+      else
+        moe_gemm_mfma_splitk_kernel<float><<<gk, 256, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, tile_expert, (float*)C, N, K, act);
+      return ta_check_launch("ta_moe_gemm");
+    }
+    dim3 g((N + 255) / 256, (tiles + 3) / 4);
     if (out_dtype == TA_BF16)
-      moe_gemm_mfma_kernel<bf16_t><<<g, 256, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, tile_expert, (bf16_t*)C, N, K, act);
+      moe_gemm_mfma_kernel<bf16_t><<<g, 256, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, tile_expert, tiles, (bf16_t*)C, N, K, act);
     else if (out_dtype == TA_F32)
-      moe_gemm_mfma_kernel<float><<<g, 256, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, tile_expert, (float*)C, N, K, act);
+      moe_gemm_mfma_kernel<float><<<g, 256, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, tile_expert, tiles, (float*)C, N, K, act);
     else
       return ta_fail("ta_moe_gemm: unknown output type %d", out_dtype);
     return ta_check_launch("ta_moe_gemm");

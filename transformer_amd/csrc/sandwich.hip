@@ -23,13 +23,82 @@ __device__ __forceinline__ float block_sum4(float v, float* red) {
 }
 
 template <typename TO>
+__device__ __forceinline__ void store4(TO* p, float a, float b, float c, float d);
+template <>
+__device__ __forceinline__ void store4<float>(float* p, float a, float b, float c, float d) {
+  *reinterpret_cast<float4*>(p) = float4{a, b, c, d};
+}
+template <>
+__device__ __forceinline__ void store4<bf16_t>(bf16_t* p, float a, float b, float c, float d) {
+  *reinterpret_cast<uint2*>(p) = uint2{f32x2_to_bf16x2_bits(a, b), f32x2_to_bf16x2_bits(c, d)};
+}
+
+// VEC: d % 4 == 0 and a thread owns runs of four columns, kept in registers (rows of up to
+// 4 * 256 * VMAX columns); else the row waits in LDS between the passes.
+template <typename TO, bool VEC>
 __global__ __launch_bounds__(256) void postnorm_add_kernel(
     float* __restrict__ x, const float* __restrict__ delta, int planes, size_t plane,
     const float* __restrict__ w, float eps, TO* __restrict__ xcast, const float* __restrict__ w_next,
     float eps_next, TO* __restrict__ out, int d) {
-  extern __shared__ float row[];          // [d]
+  extern __shared__ float row[];          // [d] (not VEC)
   __shared__ float red[4];
   const size_t base = (size_t)blockIdx.x * d;
+  if (VEC) {
+    constexpr int VMAX = 4;
+    float4 v[VMAX], xv[VMAX], wv[VMAX];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < VMAX; ++i) {
+      const int c = 4 * (threadIdx.x + 256 * i);
+      if (c < d) {
+        v[i] = *reinterpret_cast<const float4*>(delta + base + c);
+        xv[i] = *reinterpret_cast<const float4*>(x + base + c);
+        wv[i] = *reinterpret_cast<const float4*>(w + c);
+      } else {
+        v[i] = xv[i] = wv[i] = float4{0.f, 0.f, 0.f, 0.f};
+      }
+    }
+    for (int p = 1; p < planes; ++p)
+#pragma unroll
+      for (int i = 0; i < VMAX; ++i) {
+        const int c = 4 * (threadIdx.x + 256 * i);
+        if (c < d) {
+          const float4 a = *reinterpret_cast<const float4*>(delta + base + c + p * plane);
+          v[i].x += a.x; v[i].y += a.y; v[i].z += a.z; v[i].w += a.w;
+        }
+      }
+#pragma unroll
+    for (int i = 0; i < VMAX; ++i) ss += (v[i].x * v[i].x + v[i].y * v[i].y) + (v[i].z * v[i].z + v[i].w * v[i].w);
+    const float f = rsqrtf(block_sum4(ss, red) / (float)d + eps);
+    float s2 = 0.f;
+#pragma unroll
+    for (int i = 0; i < VMAX; ++i) {
+      const int c = 4 * (threadIdx.x + 256 * i);
+      v[i].x = xv[i].x + v[i].x * f * wv[i].x;
+      v[i].y = xv[i].y + v[i].y * f * wv[i].y;
+      v[i].z = xv[i].z + v[i].z * f * wv[i].z;
+      v[i].w = xv[i].w + v[i].w * f * wv[i].w;
+      if (c < d) {
+        *reinterpret_cast<float4*>(x + base + c) = v[i];
+        if (xcast) store4<TO>(xcast + base + c, v[i].x, v[i].y, v[i].z, v[i].w);
+        s2 += (v[i].x * v[i].x + v[i].y * v[i].y) + (v[i].z * v[i].z + v[i].w * v[i].w);
+      }
+    }
+    if (!out) return;
+#pragma unroll
+    for (int i = 0; i < VMAX; ++i) {
+      const int c = 4 * (threadIdx.x + 256 * i);
+      if (c < d) wv[i] = *reinterpret_cast<const float4*>(w_next + c);
+    }
+    const float f2 = rsqrtf(block_sum4(s2, red) / (float)d + eps_next);
+#pragma unroll
+    for (int i = 0; i < VMAX; ++i) {
+      const int c = 4 * (threadIdx.x + 256 * i);
+      if (c < d) store4<TO>(out + base + c, v[i].x * f2 * wv[i].x, v[i].y * f2 * wv[i].y, v[i].z * f2 * wv[i].z,
+                            v[i].w * f2 * wv[i].w);
+    }
+    return;
+  }
   float ss = 0.f;
   for (int c = threadIdx.x; c < d; c += 256) {
     float s = delta[base + c];
@@ -62,14 +131,16 @@ extern "C" int ta_postnorm_add(hipStream_t stream, int out_dtype, float* x, cons
   TA_REQUIRE((out == nullptr) == (w_next == nullptr), "ta_postnorm_add: w_next and out go together");
   if (nt == 0) return 0;
   const size_t lds = (size_t)d * sizeof(float);
-  if (out_dtype == TA_F32)
-    postnorm_add_kernel<float><<<nt, 256, lds, stream>>>(x, delta, planes, (size_t)plane, w, eps, (float*)xcast,
-                                                        w_next, eps_next, (float*)out, d);
-  else if (out_dtype == TA_BF16)
-    postnorm_add_kernel<bf16_t><<<nt, 256, lds, stream>>>(x, delta, planes, (size_t)plane, w, eps,
-                                                         (bf16_t*)xcast, w_next, eps_next, (bf16_t*)out, d);
-  else
+  const bool vec = d % 4 == 0 && d <= 4096 && plane % 4 == 0;
+#define PN_RUN(T, V, L) postnorm_add_kernel<T, V><<<nt, 256, L, stream>>>(x, delta, planes, (size_t)plane, w, eps, (T*)xcast, w_next, eps_next, (T*)out, d)
+  if (out_dtype == TA_F32) {
+    if (vec) PN_RUN(float, true, 0); else PN_RUN(float, false, lds);
+  } else if (out_dtype == TA_BF16) {
+    if (vec) PN_RUN(bf16_t, true, 0); else PN_RUN(bf16_t, false, lds);
+  } else {
     return ta_fail("ta_postnorm_add: unknown dtype %d", out_dtype);
+  }
+#undef PN_RUN
   return ta_check_launch("ta_postnorm_add");
 }
 
