@@ -236,6 +236,7 @@ union MoeFrag {
   moe_bf16x8 v;
   moe_u32x4 q;
 };
+static __device__ __forceinline__ moe_u32x4 moe_zero4() { return moe_u32x4{0, 0, 0, 0}; }
 
 // Matrix cores: a workgroup of 4 waves owns four neighbouring tiles of 16 rows, a wave 64
 // columns of them (four 16 x 16 tiles). Neighbouring tiles of one expert form a run; a wave
@@ -265,29 +266,48 @@ __device__ __forceinline__ void moe_run(const bf16_t* __restrict__ A, const bf16
   for (int u = 0; u < RUN; ++u)
 #pragma unroll
     for (int t = 0; t < 4; ++t) acc[u][t] = moe_floatx4{0.f, 0.f, 0.f, 0.f};
-  const moe_u32x4 zero = {0, 0, 0, 0};
-  MoeFrag af[RUN], wf[4], an[RUN], wn[4];
-  auto load = [&](MoeFrag* a, MoeFrag* w, int k0) {
-    const bool kok = k0 + kb * 8 < K;
-#pragma unroll
-    for (int u = 0; u < RUN; ++u) a[u].q = kok ? *reinterpret_cast<const moe_u32x4*>(arow[u] + k0) : zero;
-#pragma unroll
-    for (int t = 0; t < 4; ++t)
-      w[t].q = (kok && wok[t]) ? __builtin_nontemporal_load(reinterpret_cast<const moe_u32x4*>(wrow[t] + k0)) : zero;
+  // Three steps of 32 k are on their way while one is multiplied: a trip to memory takes several
+  // times as long as a step's products. The whole steps load without a condition (a column past
+  // N reads row 0 of the matrix and is never stored): a value chosen after its load would be
+  // waited for where the load is issued.
+  struct Step {
+    MoeFrag a[RUN], w[4];
   };
-  load(af, wf, 0);
-  for (int k0 = 0; k0 < K; k0 += 32) {
-    if (k0 + 32 < K) load(an, wn, k0 + 32);
+  auto load = [&](Step& s, int k0) {
+#pragma unroll
+    for (int u = 0; u < RUN; ++u) s.a[u].q = *reinterpret_cast<const moe_u32x4*>(arow[u] + k0);
+#pragma unroll
+    for (int t = 0; t < 4; ++t) s.w[t].q = *reinterpret_cast<const moe_u32x4*>(wrow[t] + k0);   // other tiles read it again: it stays cached
+  };
+  auto mma = [&](const Step& s) {
 #pragma unroll
     for (int t = 0; t < 4; ++t)
 #pragma unroll
       for (int u = 0; u < RUN; ++u)
         // register j of a lane: W row 4 * (lane / 16) + j of the tile, activation row lane % 16
-        acc[u][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[t].v, af[u].v, acc[u][t], 0, 0, 0);
+        acc[u][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(s.w[t].v, s.a[u].v, acc[u][t], 0, 0, 0);
+  };
+  const int KF = K / 32 * 32;                           // whole steps
+  Step s0, s1, s2;
+  if (KF > 0) load(s0, 0);
+  if (KF > 32) load(s1, 32);
+  for (int k0 = 0; k0 < KF; k0 += 96) {
+    if (k0 + 64 < KF) load(s2, k0 + 64);
+    mma(s0);
+    if (k0 + 32 >= KF) break;
+    if (k0 + 96 < KF) load(s0, k0 + 96);
+    mma(s1);
+    if (k0 + 64 >= KF) break;
+    if (k0 + 128 < KF) load(s1, k0 + 128);
+    mma(s2);
+  }
+  if (KF < K) {                                         // the last, partial step
+    const bool kok = KF + kb * 8 < K;
 #pragma unroll
-    for (int u = 0; u < RUN; ++u) af[u] = an[u];
+    for (int u = 0; u < RUN; ++u) s0.a[u].q = kok ? *reinterpret_cast<const moe_u32x4*>(arow[u] + KF) : moe_zero4();
 #pragma unroll
-    for (int t = 0; t < 4; ++t) wf[t] = wn[t];
+    for (int t = 0; t < 4; ++t) s0.w[t].q = kok ? *reinterpret_cast<const moe_u32x4*>(wrow[t] + KF) : moe_zero4();
+    mma(s0);
   }
 #pragma unroll
   for (int u = 0; u < RUN; ++u)
@@ -354,7 +374,6 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_splitk_kernel(const bf16_t*
   moe_floatx4 acc[4];
 #pragma unroll
   for (int t = 0; t < 4; ++t) acc[t] = moe_floatx4{0.f, 0.f, 0.f, 0.f};
-  const moe_u32x4 zero = {0, 0, 0, 0};
   constexpr int DEPTH = 4;                              // steps of 32 k asked for together
   for (int k0 = kbeg; k0 < kend; k0 += 32 * DEPTH) {
     MoeFrag af[DEPTH], wf[DEPTH][4];
@@ -362,10 +381,10 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_splitk_kernel(const bf16_t*
     for (int u = 0; u < DEPTH; ++u) {
       const int k = k0 + 32 * u;
       const bool kok = k < kend && k + kb * 8 < K;
-      af[u].q = kok ? *reinterpret_cast<const moe_u32x4*>(arow + k) : zero;
+      af[u].q = kok ? *reinterpret_cast<const moe_u32x4*>(arow + k) : moe_zero4();
 #pragma unroll
       for (int t = 0; t < 4; ++t)
-        wf[u][t].q = (kok && wok[t]) ? __builtin_nontemporal_load(reinterpret_cast<const moe_u32x4*>(wrow[t] + k)) : zero;
+        wf[u][t].q = (kok && wok[t]) ? __builtin_nontemporal_load(reinterpret_cast<const moe_u32x4*>(wrow[t] + k)) : moe_zero4();
     }
 #pragma unroll
     for (int u = 0; u < DEPTH; ++u)
@@ -433,15 +452,20 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
                                                           const float* __restrict__ shared, int planes, size_t plane,
                                                           const float* __restrict__ shared_gate, int gate_ld,
                                                           float* __restrict__ delta) {
+  extern __shared__ float cmb[];          // [top] rows of the token's pairs, [top] their weights
+  int* prow = reinterpret_cast<int*>(cmb);
+  float* pw = cmb + top;
   const size_t t = blockIdx.x;
+  for (int j = threadIdx.x; j < top; j += 256) {
+    prow[j] = pair_row[t * top + j];
+    pw[j] = weight ? weight[t * top + j] : 1.f;
+  }
   float sg = 1.f;
   if (shared && shared_gate) sg = 1.0f / (1.0f + expf(-shared_gate[t * gate_ld]));
+  __syncthreads();
   for (int c = threadIdx.x; c < d; c += 256) {
     float s = 0.f;
-    for (int j = 0; j < top; ++j) {
-      const float v = rows[(size_t)pair_row[t * top + j] * d + c];
-      s += weight ? v * weight[t * top + j] : v;
-    }
+    for (int j = 0; j < top; ++j) s = fmaf(rows[(size_t)prow[j] * d + c], pw[j], s);
     if (shared) {
       float v = shared[t * d + c];
       for (int p = 1; p < planes; ++p) v += shared[t * d + c + p * plane];
@@ -460,7 +484,7 @@ extern "C" int ta_moe_combine(hipStream_t stream, const float* rows, int d, int 
                               const float* shared_gate, int gate_ld, float* delta, int nt) {
   TA_REQUIRE(nt >= 0 && d > 0 && top >= 1 && planes >= 1 && planes <= TA_MAX_PLANES, "ta_moe_combine: bad sizes");
   if (nt == 0) return 0;
-  moe_combine_kernel<<<nt, 256, 0, stream>>>(rows, d, top, pair_row, weight, shared, planes, (size_t)plane,
+  moe_combine_kernel<<<nt, 256, (size_t)2 * top * sizeof(float), stream>>>(rows, d, top, pair_row, weight, shared, planes, (size_t)plane,
                                              shared_gate, gate_ld, delta);
   return ta_check_launch("ta_moe_combine");
 }
