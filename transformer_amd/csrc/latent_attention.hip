@@ -22,6 +22,7 @@
 // the one rounding of each result is float32. Keys are walked in chunks of 32 aligned to
 // absolute positions, so a row's bits depend on its own query and keys only.
 #include "common.h"
+#include <type_traits>
 
 __device__ __forceinline__ float la_block_sum(float v, float* red) {
   v = wave_sum(v);
@@ -317,7 +318,7 @@ union LaFrag {
 };
 
 template <int KS, int CT, int RT>
-__global__ __launch_bounds__(256, (KS <= 6 ? 2 : 1)) void latent_attention_mfma_kernel(
+__global__ __launch_bounds__(256, ((KS <= 6 && RT == 1) ? 2 : 1)) void latent_attention_mfma_kernel(
     const bf16_t* __restrict__ qa, bf16_t* __restrict__ out, const bf16_t* __restrict__ kcache,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ cu_q,
     const int* __restrict__ pos0, int H, int rank, int dc, float scale_log2, int window,
@@ -361,11 +362,16 @@ __global__ __launch_bounds__(256, (KS <= 6 ? 2 : 1)) void latent_attention_mfma_
   const int c0 = tile_start / 32, c1 = (tile_end + 31) / 32;
   const int n = c1 - c0;
   const int ca = c0 + (int)((long long)n * split / splits), cb = c0 + (int)((long long)n * (split + 1) / splits);
-  la_floatx4 O[RT][CT];
+  // TWO: rows too wide for one wave's registers go over the keys three times: once for every
+  // row's maximum and sum of weights, then once for each half of the coordinates, with the
+  // final maximum as the exponentials' reference, so nothing is ever rescaled.
+  constexpr bool TWO = KS > 10;
+  constexpr int CTP = TWO ? CT / 2 : CT;                  // coordinate tiles a pass sums
+  la_floatx4 O[RT][CTP];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-    for (int ct = 0; ct < CT; ++ct) O[rt][ct] = la_floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int ct = 0; ct < CTP; ++ct) O[rt][ct] = la_floatx4{0.f, 0.f, 0.f, 0.f};
   float m[RT], l[RT];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) { m[rt] = -INFINITY; l[rt] = 0.f; }
@@ -376,7 +382,8 @@ __global__ __launch_bounds__(256, (KS <= 6 ? 2 : 1)) void latent_attention_mfma_
   constexpr int NL = 2 * KS;
   constexpr bool PRE = KS <= 10;
   uint4 pre[PRE ? NL : 1];
-  auto fetch = [&](int ch, uint4* buf, int i0, int i1) {
+  auto fetch = [&](int ch, uint4* buf, auto I0, auto I1) {
+    constexpr int i0 = decltype(I0)::value, i1 = decltype(I1)::value;
     const int key0 = ch * 32;
     const size_t page = (size_t)table[key0 / TA_PAGE];
     const bf16_t* src = kcache + (page * TA_PAGE + key0 % TA_PAGE) * (size_t)dc;
@@ -389,7 +396,8 @@ __global__ __launch_bounds__(256, (KS <= 6 ? 2 : 1)) void latent_attention_mfma_
       buf[i - i0] = live ? v : uint4{0, 0, 0, 0};
     }
   };
-  auto stash = [&](const uint4* buf, int i0, int i1) {
+  auto stash = [&](const uint4* buf, auto I0, auto I1) {
+    constexpr int i0 = decltype(I0)::value, i1 = decltype(I1)::value;
 #pragma unroll
     for (int i = i0; i < i1; ++i) {
       const int idx = lane + 64 * i;
@@ -397,20 +405,36 @@ __global__ __launch_bounds__(256, (KS <= 6 ? 2 : 1)) void latent_attention_mfma_
       if (idx < 32 * pieces) *reinterpret_cast<uint4*>(Ks + k * RS + pc * 8) = buf[i - i0];
     }
   };
-  if (PRE && ca < cb) fetch(ca, pre, 0, NL);
+  using la_i0 = std::integral_constant<int, 0>;
+  using la_nl = std::integral_constant<int, NL>;
+  constexpr int NB = 12;                                  // pieces a lane brings in together without PRE
+  // MODE 2: one pass (maxima move, sums are rescaled); 0: maxima and sums of weights only; 1: the
+  // weighted sums of coordinate blocks QB0 .. with the maxima that pass 0 found.
+  auto walk = [&](auto MODE_, auto QB0_) {
+  constexpr int MODE = decltype(MODE_)::value, QB0 = decltype(QB0_)::value;
+  if (PRE && ca < cb) fetch(ca, pre, la_i0{}, la_nl{});
   for (int ch = ca; ch < cb; ++ch) {
     const int key0 = ch * 32;
     __builtin_amdgcn_wave_barrier();                      // the chunk before has been read
     if (PRE) {
-      stash(pre, 0, NL);
-      if (ch + 1 < cb) fetch(ch + 1, pre, 0, NL);
+      stash(pre, la_i0{}, la_nl{});
+      if (ch + 1 < cb) fetch(ch + 1, pre, la_i0{}, la_nl{});
     } else {
-#pragma unroll
-      for (int i0 = 0; i0 < NL; i0 += 12) {
-        uint4 buf[12];
-        fetch(ch, buf, i0, i0 + 12 < NL ? i0 + 12 : NL);
-        stash(buf, i0, i0 + 12 < NL ? i0 + 12 : NL);
-      }
+      uint4 buf[NB];
+      using b0 = std::integral_constant<int, 0>;
+      using b1 = std::integral_constant<int, (NB < NL ? NB : NL)>;
+      using b2 = std::integral_constant<int, (2 * NB < NL ? 2 * NB : NL)>;
+      using b3 = std::integral_constant<int, (3 * NB < NL ? 3 * NB : NL)>;
+      static_assert(3 * NB >= NL, "three batches cover a chunk");
+      fetch(ch, buf, b0{}, b1{});
+      stash(buf, b0{}, b1{});
+      __builtin_amdgcn_sched_barrier(0);
+      fetch(ch, buf, b1{}, b2{});
+      stash(buf, b1{}, b2{});
+      __builtin_amdgcn_sched_barrier(0);
+      fetch(ch, buf, b2{}, b3{});
+      stash(buf, b2{}, b3{});
+      __builtin_amdgcn_sched_barrier(0);
     }
     __builtin_amdgcn_wave_barrier();
     // ---- scores: register j of tile t of a lane is key 16 t + 4 g + j for the lane's row c
@@ -430,6 +454,7 @@ __global__ __launch_bounds__(256, (KS <= 6 ? 2 : 1)) void latent_attention_mfma_
         for (int rt = 0; rt < RT; ++rt)
           S[rt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qf[rt][ks].v, S[rt][t], 0, 0, 0);
       }
+      if (KS > 10 && ks % 3 == 2) __builtin_amdgcn_sched_barrier(0);    // wide rows: operands are not all asked for at once
     }
     // ---- softmax of the lane's rows over the chunk, in the log2 domain
     LaFrag pf[RT][3];
@@ -446,7 +471,7 @@ __global__ __launch_bounds__(256, (KS <= 6 ? 2 : 1)) void latent_attention_mfma_
       }
       mx = fmaxf(mx, __shfl_xor(mx, 16, TA_WAVE));
       mx = fmaxf(mx, __shfl_xor(mx, 32, TA_WAVE));
-      const float m_new = fmaxf(m[rt], mx);
+      const float m_new = MODE == 1 ? m[rt] : fmaxf(m[rt], mx);
       const float m_use = m_new == -INFINITY ? 0.f : m_new;
       const float alpha = __builtin_amdgcn_exp2f(m[rt] - m_use);       // m = -inf gives 0
       float rs = 0.f;
@@ -454,29 +479,34 @@ __global__ __launch_bounds__(256, (KS <= 6 ? 2 : 1)) void latent_attention_mfma_
       for (int e = 0; e < 8; ++e) {
         const float p = __builtin_amdgcn_exp2f(sv[e] - m_use);          // -inf gives 0
         rs += p;
-        const float r1 = p - to_f32(from_f32<bf16_t>(p));
-        const float r2 = r1 - to_f32(from_f32<bf16_t>(r1));
-        pf[rt][0].s[e] = f32_to_bf16_bits(p);
-        pf[rt][1].s[e] = f32_to_bf16_bits(r1);
-        pf[rt][2].s[e] = f32_to_bf16_bits(r2);
+        if (MODE != 0) {
+          const float r1 = p - to_f32(from_f32<bf16_t>(p));
+          const float r2 = r1 - to_f32(from_f32<bf16_t>(r1));
+          pf[rt][0].s[e] = f32_to_bf16_bits(p);
+          pf[rt][1].s[e] = f32_to_bf16_bits(r1);
+          pf[rt][2].s[e] = f32_to_bf16_bits(r2);
+        }
       }
-      rs += __shfl_xor(rs, 16, TA_WAVE);
-      rs += __shfl_xor(rs, 32, TA_WAVE);
-      l[rt] = l[rt] * alpha + rs;
-      m[rt] = m_new;
-      if (__any(alpha != 1.f)) {
+      if (MODE != 1) {
+        rs += __shfl_xor(rs, 16, TA_WAVE);
+        rs += __shfl_xor(rs, 32, TA_WAVE);
+        l[rt] = l[rt] * alpha + rs;
+        m[rt] = m_new;
+      }
+      if (MODE == 2 && __any(alpha != 1.f)) {
 #pragma unroll
-        for (int ct = 0; ct < CT; ++ct)
+        for (int ct = 0; ct < CTP; ++ct)
 #pragma unroll
           for (int j = 0; j < 4; ++j) O[rt][ct][j] *= alpha;
       }
     }
+    if (MODE == 0) continue;
     // ---- weighted sums. A lane reads 4 neighbouring coordinates (8 bytes) of each of its 8
     // keys and feeds four products from them: in product q of a block of 64 coordinates row i
     // of the first operand stands for coordinate 4 i + q, so register j of O[4 qb + q] is
     // coordinate 64 qb + 16 g + 4 j + q of the lane's row c.
 #pragma unroll
-    for (int qb = 0; qb < CT / 4; ++qb) {
+    for (int qb = QB0; qb < QB0 + CTP / 4; ++qb) {
       if (64 * qb >= rank) break;
       int col = 64 * qb + 4 * c;
       if (col > RS - 4) col = RS - 4;                     // past the row: coordinates nobody stores
@@ -496,12 +526,14 @@ __global__ __launch_bounds__(256, (KS <= 6 ? 2 : 1)) void latent_attention_mfma_
         for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
           for (int sp = 0; sp < 3; ++sp)
-            O[rt][4 * qb + q] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[rt][sp].v, O[rt][4 * qb + q], 0, 0, 0);
+            O[rt][4 * (qb - QB0) + q] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[rt][sp].v, O[rt][4 * (qb - QB0) + q], 0, 0, 0);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
   }
-  // ---- results: register j of O[4 qb + q] is coordinate 64 qb + 16 g + 4 j + q of the lane's row c
+  };
+  // ---- results: register j of O[4 (qb - QB0) + q] is coordinate 64 qb + 16 g + 4 j + q of the lane's row c
+  auto emit = [&](int qb0) {
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
     if (!ok[rt]) continue;
@@ -509,10 +541,10 @@ __global__ __launch_bounds__(256, (KS <= 6 ? 2 : 1)) void latent_attention_mfma_
     if (splits > 1) {
       float* dst = partial + ((((size_t)b * tiles_max + tile) * splits + split) * (16 * RT) + 16 * rt + c) * (rank + 2);
 #pragma unroll
-      for (int ct = 0; ct < CT; ++ct)
+      for (int ct = 0; ct < CTP; ++ct)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          const int coord = 64 * (ct / 4) + 16 * g + 4 * j + (ct % 4);
+          const int coord = 64 * (qb0 + ct / 4) + 16 * g + 4 * j + (ct % 4);
           if (coord < rank) dst[coord] = O[rt][ct][j];
         }
       if (g == 0) { dst[rank] = m[rt]; dst[rank + 1] = l[rt]; }
@@ -525,12 +557,31 @@ __global__ __launch_bounds__(256, (KS <= 6 ? 2 : 1)) void latent_attention_mfma_
     }
     bf16_t* o = out + ((size_t)q0 * H + row) * rank;
 #pragma unroll
-    for (int ct = 0; ct < CT; ++ct)
+    for (int ct = 0; ct < CTP; ++ct)
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const int coord = 64 * (ct / 4) + 16 * g + 4 * j + (ct % 4);
+        const int coord = 64 * (qb0 + ct / 4) + 16 * g + 4 * j + (ct % 4);
         if (coord < rank) o[coord] = from_f32<bf16_t>(O[rt][ct][j] * f);
       }
+  }
+  };
+  using la_c0 = std::integral_constant<int, 0>;
+  using la_c1 = std::integral_constant<int, 1>;
+  using la_c2 = std::integral_constant<int, 2>;
+  using la_half = std::integral_constant<int, CTP / 4>;
+  if (!TWO) {
+    walk(la_c2{}, la_c0{});
+    emit(0);
+  } else {
+    walk(la_c0{}, la_c0{});
+    walk(la_c1{}, la_c0{});
+    emit(0);
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int ct = 0; ct < CTP; ++ct) O[rt][ct] = la_floatx4{0.f, 0.f, 0.f, 0.f};
+    walk(la_c1{}, la_half{});
+    emit(CTP / 4);
   }
 }
 
