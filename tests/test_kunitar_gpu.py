@@ -187,6 +187,33 @@ def test_routed_feed_forward_pieces(dtype, geom):
         _close(_np(delta), want, dtype, f"{nt} tokens")
 
 
+@pytest.mark.parametrize("form", ["split_k", "direct", "lds"])
+@pytest.mark.parametrize("geom", [(5, 3, 40, 72, 700), (3, 1, 264, 200, 300), (16, 2, 130, 136, 90), (2, 2, 64, 64, 5)])
+def test_experts_products_in_every_form(form, geom):
+    """The three bfloat16 kernels of the experts' products on the same ordered rows: runs of one to
+    many tiles per expert, an expert that nobody chose, widths that end inside tiles and steps."""
+    from transformer_amd import kernels
+    E, top, N, K, nt = geom
+    rng = np.random.default_rng(E + nt)
+    chosen = np.stack([rng.choice(E - 1 if E > 2 else E, top, replace=False) for _ in range(nt)]).astype(np.int32)
+    rows = kernels.moe_max_rows(nt * top, E)
+    row_pair = torch.empty(rows, dtype=torch.int32, device=DEV)
+    tile_expert = torch.empty(rows // 16, dtype=torch.int32, device=DEV)
+    pair_row = torch.empty(nt * top, dtype=torch.int32, device=DEV)
+    kernels.moe_plan(_t(chosen, torch.int32), E, row_pair, tile_expert, pair_row)
+    h = _bf(rng.standard_normal((nt, K)))
+    w = _bf(rng.standard_normal((E, N, K)) / np.sqrt(K))
+    a = kernels.moe_gather(_t(h, torch.bfloat16), top, row_pair, None, torch.empty(rows, K, dtype=torch.bfloat16, device=DEV))
+    for out_dtype, act in ((torch.float32, None), (torch.bfloat16, "relu2")):
+        out = torch.full((rows, N), float("nan"), dtype=out_dtype, device=DEV)
+        kernels.moe_gemm(a, _t(w, torch.bfloat16), tile_expert, out, act, form=form)
+        got = _np(out)[_np(pair_row).astype(int)].reshape(nt, top, N)
+        want = np.einsum("tk,tjnk->tjn", h, w[chosen])
+        if act:
+            want = P.relu_squared(want)
+        _close(got, want, "bfloat16" if out_dtype == torch.bfloat16 else "float32", f"{out_dtype}")
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("geom", [(3, 20, 8, 8, 48, 33), (1, 16, 16, 16, 16, 1), (5, 7, 6, 4, 19, 9), (2, 12, 8, 8, 48, None),
                                   (8, 64, 32, 32, 128, 150), (4, 16, 0, 0, 300, 70)])

@@ -10,8 +10,8 @@
 //                 acts on the expert's input
 //   moe_gemm    : C[rows of a tile] = A[rows] * W[expert of the tile]^T for all tiles, with an
 //                 optional activation; float32 chains on the vector ALU, or the matrix cores
-//                 (v_mfma_f32_16x16x32_bf16) for bfloat16, where neighbouring tiles of one
-//                 expert share every load of its matrix
+//                 (v_mfma_f32_16x16x32_bf16) for bfloat16: operands through LDS for the many
+//                 tiles of a prompt, K divided among the waves for the few of a single-token step
 //   moe_combine : delta[t] = sum of the token's pairs' rows (times the weight when it acts on
 //                 the output) + sigmoid(shared gate) * the shared expert's rows
 //
@@ -405,18 +405,193 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_splitk_kernel(const bf16_t*
   }
 }
 
+// Many tiles (a prompt): operands through LDS. A workgroup owns eight neighbouring tiles of 16
+// rows and 128 columns; the runs of one expert among them are multiplied one after the other.
+// Every thread brings whole 16-byte pieces of the rows of A and of the expert's matrix (eight
+// lanes a row: whole cache lines), a step of 64 k ahead of the one being multiplied, into one of
+// two LDS buffers (rows 72 elements apart, so that the operand reads of 16 rows meet 16
+// different bank groups); a wave multiplies 64 x 64 of the 128 x 128 (4 x 4 operand tiles: every
+// LDS read feeds four products).
+#define ML_BM 128
+#define ML_BN 128
+#define ML_BK 64
+#define ML_LD 72
+
+template <typename TC>
+__global__ __launch_bounds__(256, 2) void moe_gemm_lds_kernel(const bf16_t* __restrict__ A, const bf16_t* __restrict__ W,
+                                                           const int* __restrict__ tile_expert, int tiles, int max_rows,
+                                                           TC* __restrict__ C, int N, int K, int act) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char ml_lds[];
+  bf16_t* As = reinterpret_cast<bf16_t*>(ml_lds);                       // [2][ML_BM][ML_LD]
+  bf16_t* Ws = As + 2 * ML_BM * ML_LD;                                  // [2][ML_BN][ML_LD]
+  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+  const int r = lane % 16, kb = lane / 16, wr = wave / 2, wc = wave % 2;
+  // Which (group of eight tiles, block of 128 columns) this workgroup takes. Workgroups go to the
+  // eight XCDs in turn, and each XCD has an L2 of its own: the workgroups that one XCD gets one
+  // after the other take two neighbouring groups of tiles (mostly one expert) through all blocks
+  // of columns, block by block, so that the expert's panel of 128 columns is read from memory once
+  // for both groups and the groups' rows once for all blocks.
+  const int ncol = (N + ML_BN - 1) / ML_BN;
+  const int xcd = blockIdx.x % 8, seq = blockIdx.x / 8;
+  const int unit = (seq / (2 * ncol)) * 8 + xcd, within = seq % (2 * ncol);
+  const int group = 2 * unit + within % 2;
+  const int n0 = (within / 2) * ML_BN;
+  int t = group * 8;
+  if (t >= tiles) return;
+  const int t_end = t + 8 < tiles ? t + 8 : tiles;
+  const int nk = (K + ML_BK - 1) / ML_BK;
+  while (t < t_end) {
+    const int e = tile_expert[t];
+    if (e < 0) return;                                  // the whole workgroup: tiles past the last expert's rows
+    int run = 1;
+    while (t + run < t_end && tile_expert[t + run] == e) ++run;
+    const int R = run * MOE_TILE;
+    const size_t r0 = (size_t)t * MOE_TILE;
+    const bf16_t* We = W + (size_t)e * N * K;
+    // this thread's four pieces of A and of W in a step: row p / 8, piece p % 8, p = tid + 256 i
+    const bf16_t* asrc[4];
+    const bf16_t* wsrc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int p = tid + 256 * i, row = p / 8, pc = p % 8;
+      const size_t ar = r0 + (row < R ? row : R - 1);                   // rows past the run: read again, never stored
+      const int wn = n0 + row < N ? n0 + row : N - 1;                   // columns past N likewise
+      asrc[i] = A + ar * K + pc * 8;
+      wsrc[i] = We + (size_t)wn * K + pc * 8;
+    }
+    // Three steps' pieces wait in registers on their way from memory (a trip takes several times
+    // as long as a step's products); the barrier between steps waits for LDS traffic only, not
+    // for these loads.
+    struct Pieces {
+      moe_u32x4 a[4], w[4];
+    };
+    auto fetch = [&](Pieces& q, int step) {
+      const int k0 = step * ML_BK;
+      if (step >= nk) return;
+      if (k0 + ML_BK <= K) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          q.a[i] = *reinterpret_cast<const moe_u32x4*>(asrc[i] + k0);
+          q.w[i] = *reinterpret_cast<const moe_u32x4*>(wsrc[i] + k0);
+        }
+      } else {                                                          // the last, partial step
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const bool kok = k0 + ((tid + 256 * i) % 8) * 8 < K;
+          q.a[i] = kok ? *reinterpret_cast<const moe_u32x4*>(asrc[i] + k0) : moe_zero4();
+          q.w[i] = kok ? *reinterpret_cast<const moe_u32x4*>(wsrc[i] + k0) : moe_zero4();
+        }
+      }
+    };
+    auto stash = [&](const Pieces& q, int buf) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int p = tid + 256 * i, row = p / 8, pc = p % 8;
+        *reinterpret_cast<moe_u32x4*>(As + (buf * ML_BM + row) * ML_LD + pc * 8) = q.a[i];
+        *reinterpret_cast<moe_u32x4*>(Ws + (buf * ML_BN + row) * ML_LD + pc * 8) = q.w[i];
+      }
+    };
+    auto lds_barrier = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+    moe_floatx4 acc[4][4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) acc[u][v] = moe_floatx4{0.f, 0.f, 0.f, 0.f};
+    const bool busy = 64 * wr < R;                      // a run of at most 64 rows leaves two waves only loading
+    auto multiply = [&](int buf) {
+      if (!busy) return;
+#pragma unroll
+      for (int kk = 0; kk < ML_BK; kk += 32) {
+        MoeFrag af[4], wf[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          af[u].q = *reinterpret_cast<const moe_u32x4*>(As + (buf * ML_BM + 64 * wr + 16 * u + r) * ML_LD + kk + 8 * kb);
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+          wf[v].q = *reinterpret_cast<const moe_u32x4*>(Ws + (buf * ML_BN + 64 * wc + 16 * v + r) * ML_LD + kk + 8 * kb);
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+          for (int v = 0; v < 4; ++v)
+            // register j of a lane: column 4 * (lane / 16) + j of the tile, row lane % 16
+            acc[u][v] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[v].v, af[u].v, acc[u][v], 0, 0, 0);
+      }
+    };
+    Pieces p0, p1, p2;
+    fetch(p0, 0);
+    fetch(p1, 1);
+    fetch(p2, 2);
+    stash(p0, 0);
+    fetch(p0, 3);
+    lds_barrier();
+    // step s multiplies buffer s & 1; the pieces of step s + 1 (in set (s + 1) % 3) then go to the
+    // other buffer and their set asks for step s + 4
+    for (int step = 0; step < nk; step += 3) {
+      multiply(step & 1);
+      if (step + 1 < nk) { stash(p1, (step + 1) & 1); fetch(p1, step + 4); }
+      lds_barrier();
+      if (step + 1 >= nk) break;
+      multiply((step + 1) & 1);
+      if (step + 2 < nk) { stash(p2, (step + 2) & 1); fetch(p2, step + 5); }
+      lds_barrier();
+      if (step + 2 >= nk) break;
+      multiply((step + 2) & 1);
+      if (step + 3 < nk) { stash(p0, (step + 3) & 1); fetch(p0, step + 6); }
+      lds_barrier();
+    }
+    if (busy) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        if (64 * wr + 16 * u >= R) break;
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const int n = n0 + 64 * wc + 16 * v + 4 * kb + j;
+            if (n < N) C[(r0 + 64 * wr + 16 * u + r) * N + n] = from_f32<TC>(moe_act(act, acc[u][v][j]));
+          }
+      }
+    }
+    t += run;
+  }
+}
+
 // A: [max_rows, K] ordered rows; W: [E, N, K]; C: [max_rows, N], float32 or the type of A;
 // act: 0 none, 1 gelu, 2 gelu (tanh), 3 relu squared, 4 silu. Tiles past the last expert's
 // rows are skipped and their rows of C keep what they held.
-extern "C" int ta_moe_gemm(hipStream_t stream, int dtype, int out_dtype, const void* A, const void* W,
-                           const int* tile_expert, void* C, int max_rows, int N, int K, int act) {
+static int moe_gemm_lds_launch(hipStream_t stream, int out_dtype, const void* A, const void* W, const int* tile_expert,
+                               void* C, int max_rows, int tiles, int N, int K, int act) {
+  const size_t lds = (size_t)2 * (ML_BM + ML_BN) * ML_LD * sizeof(bf16_t);
+  const int ncol = (N + ML_BN - 1) / ML_BN, groups = (tiles + 7) / 8, units = (groups + 1) / 2;
+  dim3 g((unsigned)((units + 7) / 8 * 8 * 2 * ncol));      // see the kernel: eight XCDs take units of 2 groups x all column blocks
+#define ML_RUN(TC)                                                                                               \
+  do {                                                                                                           \
+    auto kern = moe_gemm_lds_kernel<TC>;                                                                         \
+    const hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                              \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);            \
+    if (err != hipSuccess) return ta_fail("ta_moe_gemm: %zu bytes of LDS refused (%s)", lds, hipGetErrorString(err)); \
+    kern<<<g, 256, lds, stream>>>((const bf16_t*)A, (const bf16_t*)W, tile_expert, tiles, max_rows, (TC*)C, N, K, act); \
+  } while (0)
+  if (out_dtype == TA_BF16) ML_RUN(bf16_t); else ML_RUN(float);
+#undef ML_RUN
+  return ta_check_launch("ta_moe_gemm");
+}
+
+// form: 0 = chosen by the shape; 1 = the waves divide K (few tiles); 2 = runs of tiles with operands
+// straight from memory; 3 = operands through LDS (many tiles). 1 to 3 take bfloat16 with K % 8 == 0.
+extern "C" int ta_moe_gemm_form(hipStream_t stream, int dtype, int out_dtype, const void* A, const void* W,
+                                const int* tile_expert, void* C, int max_rows, int N, int K, int act, int form) {
   TA_REQUIRE(max_rows >= 0 && max_rows % MOE_TILE == 0 && N > 0 && K > 0 && act >= 0 && act <= 4,
              "ta_moe_gemm: bad sizes rows=%d N=%d K=%d act=%d", max_rows, N, K, act);
+  TA_REQUIRE(form >= 0 && form <= 3 && (form == 0 || (dtype == TA_BF16 && K % 8 == 0)),
+             "ta_moe_gemm: form %d needs bfloat16 and K %% 8 == 0", form);
   if (max_rows == 0) return 0;
   const int tiles = max_rows / MOE_TILE;
   if (dtype == TA_BF16 && K % 8 == 0) {
     if (out_dtype != TA_BF16 && out_dtype != TA_F32) return ta_fail("ta_moe_gemm: unknown output type %d", out_dtype);
-    if ((long long)tiles * ((N + 255) / 256) < 1024) {   // too few workgroups to fill the CUs: the waves divide K
+    const bool few = (long long)tiles * ((N + 255) / 256) < 1024;
+    if (form == 3 || (form == 0 && !few)) return moe_gemm_lds_launch(stream, out_dtype, A, W, tile_expert, C, max_rows, tiles, N, K, act);
+    if (form == 1 || (form == 0 && few)) {   // too few workgroups to fill the CUs: the waves divide K
       dim3 gk((N + 63) / 64, tiles);
       if (out_dtype == TA_BF16)
         moe_gemm_mfma_splitk_kernel<bf16_t><<<gk, 256, 0, stream>>>((const bf16_t*)A, (const bf16_t*)W, tile_expert, (bf16_t*)C, N, K, act);
@@ -443,6 +618,11 @@ extern "C" int ta_moe_gemm(hipStream_t stream, int dtype, int out_dtype, const v
   else
     return ta_fail("ta_moe_gemm: unsupported types %d -> %d", dtype, out_dtype);
   return ta_check_launch("ta_moe_gemm");
+}
+
+extern "C" int ta_moe_gemm(hipStream_t stream, int dtype, int out_dtype, const void* A, const void* W,
+                           const int* tile_expert, void* C, int max_rows, int N, int K, int act) {
+  return ta_moe_gemm_form(stream, dtype, out_dtype, A, W, tile_expert, C, max_rows, N, K, act, 0);
 }
 
 // ------------------------------------------------------------------ putting the rows back

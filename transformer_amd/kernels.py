@@ -1515,18 +1515,25 @@ def moe_gather(h: torch.Tensor, top: int, row_pair: torch.Tensor, weight, out: t
     return out
 
 
+_MOE_FORMS = {"auto": 0, "split_k": 1, "direct": 2, "lds": 3}
+
+
 def moe_gemm(a: torch.Tensor, w: torch.Tensor, tile_expert: torch.Tensor, out: torch.Tensor,
-             act: Optional[str] = None) -> torch.Tensor:
+             act: Optional[str] = None, form: str = "auto") -> torch.Tensor:
     """out[rows of tile i] = act(a[rows] @ w[tile_expert[i]].T): a [rows, K], w [E, N, K], out
-    [rows, N] in a's type or float32."""
+    [rows, N] in a's type or float32. form: which bfloat16 kernel runs ("auto": the shape
+    decides between "lds", for many tiles, and "split_k", for few; "direct": operands straight
+    from memory)."""
+    if form not in _MOE_FORMS:
+        raise KernelError(f"moe_gemm: unknown form {form!r}; known: {sorted(_MOE_FORMS)}")
     _dev(a, "a"); _dev(w, "w", a.dtype); _dev(out, "out"); _dev(tile_expert, "tile_expert", torch.int32)
     rows, K = a.shape
     if act not in _MOE_ACTS or w.dim() != 3 or w.shape[2] != K or out.shape != (rows, w.shape[1]) \
             or tile_expert.numel() * 16 != rows:
         raise KernelError(f"moe_gemm: a {tuple(a.shape)} w {tuple(w.shape)} out {tuple(out.shape)} act {act!r}")
-    _check(library().ta_moe_gemm(_stream(), c_int(_code(a.dtype)), c_int(_code(out.dtype)), _ptr(a), _ptr(w),
-                                 _ptr(tile_expert), _ptr(out), c_int(rows), c_int(w.shape[1]), c_int(K),
-                                 c_int(_MOE_ACTS[act])))
+    _check(library().ta_moe_gemm_form(_stream(), c_int(_code(a.dtype)), c_int(_code(out.dtype)), _ptr(a), _ptr(w),
+                                      _ptr(tile_expert), _ptr(out), c_int(rows), c_int(w.shape[1]), c_int(K),
+                                      c_int(_MOE_ACTS[act]), c_int(_MOE_FORMS[form])))
     return out
 
 
