@@ -331,7 +331,11 @@ __global__ __launch_bounds__(256, ((KS <= 6 && RT == 1) ? 2 : 1)) void latent_at
   const int b = blockIdx.y, split = blockIdx.z;
   const int q0 = cu_q[b], qlen = cu_q[b + 1] - q0;
   const int nrows = qlen * H;
-  const int tile = blockIdx.x * 4 + wave;
+  // HALVES: rows too wide for one wave's registers (128 accumulators and 72 query registers): two
+  // waves take the same tile, form the same scores, and each sums one half of the coordinates.
+  constexpr bool HALVES = KS > 10;
+  const int wid = blockIdx.x * 4 + wave;
+  const int tile = HALVES ? wid / 2 : wid, half = HALVES ? wid % 2 : 0;
   const int row0 = tile * 16 * RT;
   if (row0 >= nrows) return;                              // a wave leaves alone: nothing below waits for others
   const int p0 = pos0[b];
@@ -362,11 +366,8 @@ __global__ __launch_bounds__(256, ((KS <= 6 && RT == 1) ? 2 : 1)) void latent_at
   const int c0 = tile_start / 32, c1 = (tile_end + 31) / 32;
   const int n = c1 - c0;
   const int ca = c0 + (int)((long long)n * split / splits), cb = c0 + (int)((long long)n * (split + 1) / splits);
-  // TWO: rows too wide for one wave's registers go over the keys three times: once for every
-  // row's maximum and sum of weights, then once for each half of the coordinates, with the
-  // final maximum as the exponentials' reference, so nothing is ever rescaled.
-  constexpr bool TWO = KS > 10;
-  constexpr int CTP = TWO ? CT / 2 : CT;                  // coordinate tiles a pass sums
+  constexpr int CTP = HALVES ? CT / 2 : CT;               // coordinate tiles this wave sums
+  const int qb0 = half * (CTP / 4);                       // its first block of 64 coordinates
   la_floatx4 O[RT][CTP];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt)
@@ -408,10 +409,6 @@ __global__ __launch_bounds__(256, ((KS <= 6 && RT == 1) ? 2 : 1)) void latent_at
   using la_i0 = std::integral_constant<int, 0>;
   using la_nl = std::integral_constant<int, NL>;
   constexpr int NB = 12;                                  // pieces a lane brings in together without PRE
-  // MODE 2: one pass (maxima move, sums are rescaled); 0: maxima and sums of weights only; 1: the
-  // weighted sums of coordinate blocks QB0 .. with the maxima that pass 0 found.
-  auto walk = [&](auto MODE_, auto QB0_) {
-  constexpr int MODE = decltype(MODE_)::value, QB0 = decltype(QB0_)::value;
   if (PRE && ca < cb) fetch(ca, pre, la_i0{}, la_nl{});
   for (int ch = ca; ch < cb; ++ch) {
     const int key0 = ch * 32;
@@ -471,7 +468,7 @@ __global__ __launch_bounds__(256, ((KS <= 6 && RT == 1) ? 2 : 1)) void latent_at
       }
       mx = fmaxf(mx, __shfl_xor(mx, 16, TA_WAVE));
       mx = fmaxf(mx, __shfl_xor(mx, 32, TA_WAVE));
-      const float m_new = MODE == 1 ? m[rt] : fmaxf(m[rt], mx);
+      const float m_new = fmaxf(m[rt], mx);
       const float m_use = m_new == -INFINITY ? 0.f : m_new;
       const float alpha = __builtin_amdgcn_exp2f(m[rt] - m_use);       // m = -inf gives 0
       float rs = 0.f;
@@ -479,34 +476,30 @@ __global__ __launch_bounds__(256, ((KS <= 6 && RT == 1) ? 2 : 1)) void latent_at
       for (int e = 0; e < 8; ++e) {
         const float p = __builtin_amdgcn_exp2f(sv[e] - m_use);          // -inf gives 0
         rs += p;
-        if (MODE != 0) {
-          const float r1 = p - to_f32(from_f32<bf16_t>(p));
-          const float r2 = r1 - to_f32(from_f32<bf16_t>(r1));
-          pf[rt][0].s[e] = f32_to_bf16_bits(p);
-          pf[rt][1].s[e] = f32_to_bf16_bits(r1);
-          pf[rt][2].s[e] = f32_to_bf16_bits(r2);
-        }
+        const float r1 = p - to_f32(from_f32<bf16_t>(p));
+        const float r2 = r1 - to_f32(from_f32<bf16_t>(r1));
+        pf[rt][0].s[e] = f32_to_bf16_bits(p);
+        pf[rt][1].s[e] = f32_to_bf16_bits(r1);
+        pf[rt][2].s[e] = f32_to_bf16_bits(r2);
       }
-      if (MODE != 1) {
-        rs += __shfl_xor(rs, 16, TA_WAVE);
-        rs += __shfl_xor(rs, 32, TA_WAVE);
-        l[rt] = l[rt] * alpha + rs;
-        m[rt] = m_new;
-      }
-      if (MODE == 2 && __any(alpha != 1.f)) {
+      rs += __shfl_xor(rs, 16, TA_WAVE);
+      rs += __shfl_xor(rs, 32, TA_WAVE);
+      l[rt] = l[rt] * alpha + rs;
+      m[rt] = m_new;
+      if (__any(alpha != 1.f)) {
 #pragma unroll
         for (int ct = 0; ct < CTP; ++ct)
 #pragma unroll
           for (int j = 0; j < 4; ++j) O[rt][ct][j] *= alpha;
       }
     }
-    if (MODE == 0) continue;
     // ---- weighted sums. A lane reads 4 neighbouring coordinates (8 bytes) of each of its 8
     // keys and feeds four products from them: in product q of a block of 64 coordinates row i
     // of the first operand stands for coordinate 4 i + q, so register j of O[4 qb + q] is
     // coordinate 64 qb + 16 g + 4 j + q of the lane's row c.
 #pragma unroll
-    for (int qb = QB0; qb < QB0 + CTP / 4; ++qb) {
+    for (int qi = 0; qi < CTP / 4; ++qi) {
+      const int qb = qb0 + qi;
       if (64 * qb >= rank) break;
       int col = 64 * qb + 4 * c;
       if (col > RS - 4) col = RS - 4;                     // past the row: coordinates nobody stores
@@ -526,14 +519,12 @@ __global__ __launch_bounds__(256, ((KS <= 6 && RT == 1) ? 2 : 1)) void latent_at
         for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
           for (int sp = 0; sp < 3; ++sp)
-            O[rt][4 * (qb - QB0) + q] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[rt][sp].v, O[rt][4 * (qb - QB0) + q], 0, 0, 0);
+            O[rt][4 * qi + q] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[rt][sp].v, O[rt][4 * qi + q], 0, 0, 0);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
   }
-  };
-  // ---- results: register j of O[4 (qb - QB0) + q] is coordinate 64 qb + 16 g + 4 j + q of the lane's row c
-  auto emit = [&](int qb0) {
+  // ---- results: register j of O[4 qi + q] is coordinate 64 (qb0 + qi) + 16 g + 4 j + q of the lane's row c
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
     if (!ok[rt]) continue;
@@ -547,7 +538,7 @@ __global__ __launch_bounds__(256, ((KS <= 6 && RT == 1) ? 2 : 1)) void latent_at
           const int coord = 64 * (qb0 + ct / 4) + 16 * g + 4 * j + (ct % 4);
           if (coord < rank) dst[coord] = O[rt][ct][j];
         }
-      if (g == 0) { dst[rank] = m[rt]; dst[rank + 1] = l[rt]; }
+      if (g == 0 && half == 0) { dst[rank] = m[rt]; dst[rank + 1] = l[rt]; }
       continue;
     }
     float f = l[rt] > 0.f ? 1.0f / l[rt] : 0.f;
@@ -563,25 +554,6 @@ __global__ __launch_bounds__(256, ((KS <= 6 && RT == 1) ? 2 : 1)) void latent_at
         const int coord = 64 * (qb0 + ct / 4) + 16 * g + 4 * j + (ct % 4);
         if (coord < rank) o[coord] = from_f32<bf16_t>(O[rt][ct][j] * f);
       }
-  }
-  };
-  using la_c0 = std::integral_constant<int, 0>;
-  using la_c1 = std::integral_constant<int, 1>;
-  using la_c2 = std::integral_constant<int, 2>;
-  using la_half = std::integral_constant<int, CTP / 4>;
-  if (!TWO) {
-    walk(la_c2{}, la_c0{});
-    emit(0);
-  } else {
-    walk(la_c0{}, la_c0{});
-    walk(la_c1{}, la_c0{});
-    emit(0);
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-      for (int ct = 0; ct < CTP; ++ct) O[rt][ct] = la_floatx4{0.f, 0.f, 0.f, 0.f};
-    walk(la_c1{}, la_half{});
-    emit(CTP / 4);
   }
 }
 
@@ -675,7 +647,8 @@ extern "C" int ta_latent_attention(hipStream_t stream, int dtype, const void* qa
     TA_REQUIRE(splits >= 1 && splits <= 65535 && (splits == 1 || scratch != nullptr), "ta_latent_attention: %d shares without scratch", splits);
     const long long tiles = ((long long)max_qlen * H + rows - 1) / rows;
     TA_REQUIRE(tiles <= 2147483647ll, "ta_latent_attention: too many rows");
-    dim3 g((unsigned)((tiles + 3) / 4), batch, splits);
+    const bool halves = !(dc <= 320 && rank <= 256);      // two waves a tile: see the kernel
+    dim3 g((unsigned)(((halves ? 2 : 1) * tiles + 3) / 4), batch, splits);
     const size_t lds = (size_t)4 * 32 * (dc + 8) * sizeof(bf16_t);
     const float sl2 = scale * 1.4426950408889634f;
     int rc;
