@@ -523,3 +523,92 @@ def test_random_weights_and_save_round_trip():
         b = again.step(cache, [Entry(cache.alloc_slot(), toks, [19])]).cpu().numpy()
     assert np.abs(a - b).max() < 1e-6 * max(1.0, np.abs(a).max())
     assert U.row_error(a, want).max() < U.TOL["float32"]
+
+
+def _draw_config(case):
+    """A random Kunitar configuration: any order of the two mixers, readers of earlier layers' rows
+    with windows of their own, every kind of feed-forward or none, sizes that are odd or no power
+    of two."""
+    r = np.random.default_rng(case)
+    width = int(r.choice([40, 66, 100, 136, 33, 257]))
+    layers, sources = [], []
+    for i in range(int(r.integers(1, 6))):
+        mlp = [None, U._dense(int(r.choice([24, 57, 130]))),
+               U._moe(int(r.choice([1, 2, 5, 9, 16])), 1, int(r.choice([8, 20, 33])),
+                      shared=None if r.integers(0, 2) else int(r.choice([6, 24])))][int(r.integers(0, 3))]
+        if mlp is not None and mlp["kind"] == "moe":
+            mlp["router"]["top"] = int(r.integers(1, mlp["router"]["experts"] + 1))
+        if r.integers(0, 2):
+            layers.append(U._wkv(int(r.choice([1, 2, 3, 5])), int(r.choice([8, 12, 20, 32, 40])), int(r.choice([1, 3, 8])), mlp))
+            continue
+        window = None if r.integers(0, 4) == 0 else int(r.choice([1, 2, 7, 31, 64, 65, 100]))
+        if sources and r.integers(0, 2):
+            j = int(r.choice(sources))
+            m = layers[j]["mixer"]
+            layers.append(U._lat(int(r.choice([1, 2, 4, 7])), int(r.choice([4, 10, 16, 24])), m["rot_dim"], int(r.choice([6, 16, 30])),
+                                 int(r.choice([8, 20, 48])), m["kv_rank"], float(r.choice([0.1, 0.25])), m["rot"]["base"],
+                                 window=window, kv_from=j, mlp=mlp, dims=m["rot"]["dims"]))
+            continue
+        rot_dim = int(r.choice([2, 4, 8, 10, 16]))
+        sources.append(i)
+        layers.append(U._lat(int(r.choice([1, 2, 3, 6])), int(r.choice([4, 10, 16, 24])), rot_dim, int(r.choice([6, 16, 30])),
+                             int(r.choice([8, 20, 48])), int(r.choice([8, 24, 40, 72])), float(r.choice([0.1, 0.25])),
+                             float(r.choice([100.0, 1e4, 5e5])), window=window, mlp=mlp,
+                             dims=rot_dim if r.integers(0, 2) else 2 * int(r.integers(1, rot_dim // 2 + 1))))
+    cfg = {"architecture": "Kunitar", "vocab": int(r.choice([5, 97, 300, 1001])), "width": width,
+           "norm": {"eps": float(r.choice([1e-6, 1e-5, 1e-3]))}, "embedding": {"scale": float(r.choice([1.0, 0.5, 3.0]))},
+           "layers": layers}
+    if r.integers(0, 3):
+        cfg["token_side"] = {"dim": int(r.choice([1, 4, 7, 16]))}
+    lens = [int(x) for x in r.integers(1, 150, size=int(r.integers(1, 5)))]
+    return cfg, lens, r
+
+
+@pytest.mark.parametrize("first", [2000, 2006, 2012])
+def test_random_configurations_against_the_plain_model(first):
+    """float32, the plain model's own routing, every row: a batch of unequal prompts in one step into
+    poisoned pages, then eight single tokens each (recorded steps)."""
+    import tempfile
+    import transformer_amd as ta
+    from gpu_util import poison
+    for case in range(first, first + 6):
+        cfg, lens, r = _draw_config(case)
+        with tempfile.TemporaryDirectory(prefix="ku_rand_") as d:
+            P.make_model_folder(d, cfg, case, storage="F32")
+            ref = P.PlainKunitar(d)
+            model = ta.load_model(d, "float32", "cuda:0")
+        toks = [[int(t) for t in r.integers(0, cfg["vocab"], size=n + 8)] for n in lens]
+        cache = model.new_cache(64 * sum(-(-(n + 8) // 64) for n in lens), max_slots=len(lens))
+        poison(cache)
+        slots = [cache.alloc_slot() for _ in lens]
+        want = [ref.forward(t) for t in toks]
+        what = f"case {case} {json.dumps(cfg)} prompts {lens}"
+        got = model.step(cache, [ta.Entry(s, t[:n], [n - 1]) for s, t, n in zip(slots, toks, lens)]).cpu().numpy()
+        for i, n in enumerate(lens):
+            assert U.row_error(got[i], want[i][n - 1]) < U.TOL["float32"], what
+        for j in range(8):
+            got = model.step(cache, [ta.Entry(s, [t[n + j]], [0]) for s, t, n in zip(slots, toks, lens)]).cpu().numpy()
+            for i, n in enumerate(lens):
+                assert U.row_error(got[i], want[i][n + j]) < U.TOL["float32"], (what, j)
+        for s in slots:
+            cache.free_slot(s)
+        cache.pool.check()
+        # the same in bfloat16 (matrix cores, odd widths): rows are finite, and all but the few that a
+        # close call between two experts moves lie within rounding of the plain model
+        with tempfile.TemporaryDirectory(prefix="ku_rand_") as d:
+            P.make_model_folder(d, cfg, case, storage="BF16")
+            model = ta.load_model(d, "bfloat16", "cuda:0")
+        cache = model.new_cache(64 * sum(-(-(n + 8) // 64) for n in lens), max_slots=len(lens))
+        poison(cache)
+        slots = [cache.alloc_slot() for _ in lens]
+        errs = []
+        got = model.step(cache, [ta.Entry(s, t[:n], list(range(n))) for s, t, n in zip(slots, toks, lens)]).cpu().numpy()
+        at = 0
+        for i, n in enumerate(lens):
+            errs += list(U.row_error(got[at:at + n], want[i][:n]))
+            at += n
+        for j in range(8):
+            got = model.step(cache, [ta.Entry(s, [t[n + j]], [0]) for s, t, n in zip(slots, toks, lens)]).cpu().numpy()
+            errs += [U.row_error(got[i], want[i][n + j]) for i, n in enumerate(lens)]
+        errs = np.asarray(errs)
+        assert np.isfinite(errs).all() and np.median(errs) < U.TOL["bfloat16"], (what, np.median(errs))

@@ -286,10 +286,12 @@ static int latent_attention_run(hipStream_t stream, dim3 g, size_t lds, const vo
                                 const int* pos0, int H, int rank, int rot, float scale, int window,
                                 const void* gate, int gate_stride, int dc) {
   auto kern = latent_attention_kernel<T, NACC>;
-  if (lds > 64 * 1024) {
+  static size_t allowed = 64 * 1024;                    // per instantiation: asked for once, not at every launch
+  if (lds > allowed) {
     const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return ta_fail("ta_latent_attention: %zu bytes of LDS refused (%s)", lds, hipGetErrorString(e));
+    allowed = lds;
   }
   kern<<<g, 256, lds, stream>>>((const T*)qa, (T*)out, (const T*)kcache, block_table, max_blocks, cu_q, pos0, H,
                                 rank, rot, scale, window, (const T*)gate, gate_stride, dc);
@@ -601,10 +603,12 @@ static int latent_mfma_run(hipStream_t stream, dim3 g, size_t lds, const void* q
                            int rank, int dc, float scale_log2, int window, const void* gate, int gate_stride,
                            int splits, int tiles_max, float* partial) {
   auto kern = latent_attention_mfma_kernel<KS, CT, RT>;
-  if (lds > 64 * 1024) {
+  static size_t allowed = 64 * 1024;                    // per instantiation: asked for once, not at every launch
+  if (lds > allowed) {
     const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return ta_fail("ta_latent_attention: %zu bytes of LDS refused (%s)", lds, hipGetErrorString(e));
+    allowed = lds;
   }
   kern<<<g, 256, lds, stream>>>((const bf16_t*)qa, (bf16_t*)out, (const bf16_t*)kcache, block_table, max_blocks,
                                 cu_q, pos0, H, rank, dc, scale_log2, window, (const bf16_t*)gate, gate_stride, splits,

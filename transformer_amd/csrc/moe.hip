@@ -567,9 +567,13 @@ static int moe_gemm_lds_launch(hipStream_t stream, int out_dtype, const void* A,
 #define ML_RUN(TC)                                                                                               \
   do {                                                                                                           \
     auto kern = moe_gemm_lds_kernel<TC>;                                                                         \
-    const hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                              \
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);            \
-    if (err != hipSuccess) return ta_fail("ta_moe_gemm: %zu bytes of LDS refused (%s)", lds, hipGetErrorString(err)); \
+    static bool allowed = false;                        /* asked for once, not at every launch */                \
+    if (!allowed) {                                                                                              \
+      const hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),                            \
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);          \
+      if (err != hipSuccess) return ta_fail("ta_moe_gemm: %zu bytes of LDS refused (%s)", lds, hipGetErrorString(err)); \
+      allowed = true;                                                                                            \
+    }                                                                                                            \
     kern<<<g, 256, lds, stream>>>((const bf16_t*)A, (const bf16_t*)W, tile_expert, tiles, max_rows, (TC*)C, N, K, act); \
   } while (0)
   if (out_dtype == TA_BF16) ML_RUN(bf16_t); else ML_RUN(float);
