@@ -266,6 +266,44 @@ def test_latent_attention_pieces(dtype, geom):
     cache.pool.check()
 
 
+@pytest.mark.parametrize("geom", [(3, 48, 8, 33), (2, 16, 0, 1), (5, 19, 6, None), (16, 128, 32, 150), (4, 300, 4, 70),
+                                  (2, 512, 64, 100), (7, 200, 64, 40)])
+def test_latent_attention_kernels_agree(geom):
+    """The matrix-core kernels (a workgroup's waves sharing their chunks, for steps of many rows; a wave
+    alone, with a row's keys dealt to one, three and seven waves) against the float32 kernel on the
+    same bfloat16 values: sequences of unequal lengths that go on from unequal starts, in pages
+    handed out in a scrambled order, with a gate."""
+    from transformer_amd import kernels
+    from transformer_amd.cache.storage import PAGE
+    H, r, dr, window = geom
+    rng = np.random.default_rng(H * 1000 + r)
+    W = kernels.latent_row_width(r, dr, torch.bfloat16)
+    starts, lens = [0, 130, 65, 7], [90, 75, 1, 140]
+    total = sum(lens)
+    npages = sum(-(-(a + n) // PAGE) for a, n in zip(starts, lens))
+    order = rng.permutation(npages)
+    table = np.zeros((len(lens), max(-(-(a + n) // PAGE) for a, n in zip(starts, lens))), dtype=np.int32)
+    at = 0
+    for i, (a, n) in enumerate(zip(starts, lens)):
+        k = -(-(a + n) // PAGE)
+        table[i, :k] = order[at:at + k]
+        at += k
+    rows = _bf(rng.standard_normal((npages + 1, 1, PAGE, W)))
+    rows[..., r + dr:] = 0.0
+    qa = _bf(2.0 * rng.standard_normal((total, H, W)))
+    qa[..., r + dr:] = 0.0
+    gate = _bf(rng.standard_normal((total, H + 3)))
+    cu = _t(np.concatenate([[0], np.cumsum(lens)]), torch.int32)
+    args = (_t(table, torch.int32), cu, _t(starts, torch.int32), max(lens), r, dr, 0.2, window)
+    want = torch.empty(total, H, r, device=DEV)
+    kernels.latent_attention(_t(qa[..., :r + dr]), want, _t(rows[..., :r + dr]), *args, gate=_t(gate)[:, 2:])
+    for shares in (1, 3, 7):
+        out = torch.full((total, H, r), float("nan"), dtype=torch.bfloat16, device=DEV)
+        kernels.latent_attention(_t(qa, torch.bfloat16), out, _t(rows, torch.bfloat16), *args,
+                                 gate=_t(gate, torch.bfloat16)[:, 2:], shares=shares)
+        _close(_np(out), _np(want), "bfloat16", f"{shares} shares")
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("where", ["prompt", "decode"])
 def test_far_key_and_window_edges_stand_out(where, dtype):

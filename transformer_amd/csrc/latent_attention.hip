@@ -319,6 +319,104 @@ union LaFrag {
   uint16_t s[8];
 };
 
+// One chunk of 32 keys, already in LDS at Ks (rows RS elements apart), for the RT tiles of a wave:
+// scores, softmax in the log2 domain, weighted sums of the coordinate blocks from qb0 on.
+template <int KS, int CTP, int RT>
+__device__ __forceinline__ void la_chunk(const bf16_t* __restrict__ Ks, int RS, int dc, int rank, int key0, int c, int g,
+                                         const LaFrag (&qf)[RT][KS], const bool (&ok)[RT], const int (&my_start)[RT],
+                                         const int (&my_end)[RT], float scale_log2, float (&m)[RT], float (&l)[RT],
+                                         la_floatx4 (&O)[RT][CTP], int qb0) {
+    // ---- scores: register j of tile t of a lane is key 16 t + 4 g + j for the lane's row c
+    la_floatx4 S[RT][2];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+      for (int t = 0; t < 2; ++t) S[rt][t] = la_floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int d = 32 * ks + 8 * g;
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        LaFrag kf;
+        kf.q = d < dc ? *reinterpret_cast<const uint4*>(Ks + (16 * t + c) * RS + d) : uint4{0, 0, 0, 0};
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+          S[rt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qf[rt][ks].v, S[rt][t], 0, 0, 0);
+      }
+      if (KS > 10 && ks % 3 == 2) __builtin_amdgcn_sched_barrier(0);    // wide rows: operands are not all asked for at once
+    }
+    // ---- softmax of the lane's rows over the chunk, in the log2 domain
+    LaFrag pf[RT][3];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+      float sv[8];
+      float mx = -INFINITY;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int key = key0 + 16 * (e / 4) + 4 * g + (e % 4);
+        const bool vis = ok[rt] && key >= my_start[rt] && key < my_end[rt];
+        sv[e] = vis ? S[rt][e / 4][e % 4] * scale_log2 : -INFINITY;
+        mx = fmaxf(mx, sv[e]);
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, TA_WAVE));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, TA_WAVE));
+      const float m_new = fmaxf(m[rt], mx);
+      const float m_use = m_new == -INFINITY ? 0.f : m_new;
+      const float alpha = __builtin_amdgcn_exp2f(m[rt] - m_use);       // m = -inf gives 0
+      float rs = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float p = __builtin_amdgcn_exp2f(sv[e] - m_use);          // -inf gives 0
+        rs += p;
+        const float r1 = p - to_f32(from_f32<bf16_t>(p));
+        const float r2 = r1 - to_f32(from_f32<bf16_t>(r1));
+        pf[rt][0].s[e] = f32_to_bf16_bits(p);
+        pf[rt][1].s[e] = f32_to_bf16_bits(r1);
+        pf[rt][2].s[e] = f32_to_bf16_bits(r2);
+      }
+      rs += __shfl_xor(rs, 16, TA_WAVE);
+      rs += __shfl_xor(rs, 32, TA_WAVE);
+      l[rt] = l[rt] * alpha + rs;
+      m[rt] = m_new;
+      if (__any(alpha != 1.f)) {
+#pragma unroll
+        for (int ct = 0; ct < CTP; ++ct)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) O[rt][ct][j] *= alpha;
+      }
+    }
+    // ---- weighted sums. A lane reads 4 neighbouring coordinates (8 bytes) of each of its 8
+    // keys and feeds four products from them: in product q of a block of 64 coordinates row i
+    // of the first operand stands for coordinate 4 i + q, so register j of O[4 qb + q] is
+    // coordinate 64 qb + 16 g + 4 j + q of the lane's row c.
+#pragma unroll
+    for (int qi = 0; qi < CTP / 4; ++qi) {
+      const int qb = qb0 + qi;
+      if (64 * qb >= rank) break;
+      int col = 64 * qb + 4 * c;
+      if (col > RS - 4) col = RS - 4;                     // past the row: coordinates nobody stores
+      uint2 wv[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        wv[e] = *reinterpret_cast<const uint2*>(Ks + (16 * (e / 4) + 4 * g + (e % 4)) * RS + col);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        LaFrag vf;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const uint32_t lo = q < 2 ? wv[2 * i].x : wv[2 * i].y, hi = q < 2 ? wv[2 * i + 1].x : wv[2 * i + 1].y;
+          vf.w[i] = __builtin_amdgcn_perm(hi, lo, (q & 1) ? 0x07060302u : 0x05040100u);
+        }
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+          for (int sp = 0; sp < 3; ++sp)
+            O[rt][4 * qi + q] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[rt][sp].v, O[rt][4 * qi + q], 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+
 template <int KS, int CT, int RT>
 __global__ __launch_bounds__(256, ((KS <= 6 && RT == 1) ? 2 : 1)) void latent_attention_mfma_kernel(
     const bf16_t* __restrict__ qa, bf16_t* __restrict__ out, const bf16_t* __restrict__ kcache,
@@ -436,95 +534,7 @@ __global__ __launch_bounds__(256, ((KS <= 6 && RT == 1) ? 2 : 1)) void latent_at
       __builtin_amdgcn_sched_barrier(0);
     }
     __builtin_amdgcn_wave_barrier();
-    // ---- scores: register j of tile t of a lane is key 16 t + 4 g + j for the lane's row c
-    la_floatx4 S[RT][2];
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-      for (int t = 0; t < 2; ++t) S[rt][t] = la_floatx4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      const int d = 32 * ks + 8 * g;
-#pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        LaFrag kf;
-        kf.q = d < dc ? *reinterpret_cast<const uint4*>(Ks + (16 * t + c) * RS + d) : uint4{0, 0, 0, 0};
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt)
-          S[rt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qf[rt][ks].v, S[rt][t], 0, 0, 0);
-      }
-      if (KS > 10 && ks % 3 == 2) __builtin_amdgcn_sched_barrier(0);    // wide rows: operands are not all asked for at once
-    }
-    // ---- softmax of the lane's rows over the chunk, in the log2 domain
-    LaFrag pf[RT][3];
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt) {
-      float sv[8];
-      float mx = -INFINITY;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const int key = key0 + 16 * (e / 4) + 4 * g + (e % 4);
-        const bool vis = ok[rt] && key >= my_start[rt] && key < my_end[rt];
-        sv[e] = vis ? S[rt][e / 4][e % 4] * scale_log2 : -INFINITY;
-        mx = fmaxf(mx, sv[e]);
-      }
-      mx = fmaxf(mx, __shfl_xor(mx, 16, TA_WAVE));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, TA_WAVE));
-      const float m_new = fmaxf(m[rt], mx);
-      const float m_use = m_new == -INFINITY ? 0.f : m_new;
-      const float alpha = __builtin_amdgcn_exp2f(m[rt] - m_use);       // m = -inf gives 0
-      float rs = 0.f;
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const float p = __builtin_amdgcn_exp2f(sv[e] - m_use);          // -inf gives 0
-        rs += p;
-        const float r1 = p - to_f32(from_f32<bf16_t>(p));
-        const float r2 = r1 - to_f32(from_f32<bf16_t>(r1));
-        pf[rt][0].s[e] = f32_to_bf16_bits(p);
-        pf[rt][1].s[e] = f32_to_bf16_bits(r1);
-        pf[rt][2].s[e] = f32_to_bf16_bits(r2);
-      }
-      rs += __shfl_xor(rs, 16, TA_WAVE);
-      rs += __shfl_xor(rs, 32, TA_WAVE);
-      l[rt] = l[rt] * alpha + rs;
-      m[rt] = m_new;
-      if (__any(alpha != 1.f)) {
-#pragma unroll
-        for (int ct = 0; ct < CTP; ++ct)
-#pragma unroll
-          for (int j = 0; j < 4; ++j) O[rt][ct][j] *= alpha;
-      }
-    }
-    // ---- weighted sums. A lane reads 4 neighbouring coordinates (8 bytes) of each of its 8
-    // keys and feeds four products from them: in product q of a block of 64 coordinates row i
-    // of the first operand stands for coordinate 4 i + q, so register j of O[4 qb + q] is
-    // coordinate 64 qb + 16 g + 4 j + q of the lane's row c.
-#pragma unroll
-    for (int qi = 0; qi < CTP / 4; ++qi) {
-      const int qb = qb0 + qi;
-      if (64 * qb >= rank) break;
-      int col = 64 * qb + 4 * c;
-      if (col > RS - 4) col = RS - 4;                     // past the row: coordinates nobody stores
-      uint2 wv[8];
-#pragma unroll
-      for (int e = 0; e < 8; ++e)
-        wv[e] = *reinterpret_cast<const uint2*>(Ks + (16 * (e / 4) + 4 * g + (e % 4)) * RS + col);
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        LaFrag vf;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const uint32_t lo = q < 2 ? wv[2 * i].x : wv[2 * i].y, hi = q < 2 ? wv[2 * i + 1].x : wv[2 * i + 1].y;
-          vf.w[i] = __builtin_amdgcn_perm(hi, lo, (q & 1) ? 0x07060302u : 0x05040100u);
-        }
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-          for (int sp = 0; sp < 3; ++sp)
-            O[rt][4 * qi + q] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf[rt][sp].v, O[rt][4 * qi + q], 0, 0, 0);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-    }
+    la_chunk<KS, CTP, RT>(Ks, RS, dc, rank, key0, c, g, qf, ok, my_start, my_end, scale_log2, m, l, O, qb0);
   }
   // ---- results: register j of O[4 qi + q] is coordinate 64 (qb0 + qi) + 16 g + 4 j + q of the lane's row c
 #pragma unroll
@@ -557,6 +567,162 @@ __global__ __launch_bounds__(256, ((KS <= 6 && RT == 1) ? 2 : 1)) void latent_at
         if (coord < rank) o[coord] = from_f32<bf16_t>(O[rt][ct][j] * f);
       }
   }
+}
+
+// Steps of many rows (prompts): the four waves of a workgroup own four neighbouring tiles of 16
+// rows, whose key ranges all but coincide, and SHARE every chunk: 256 threads bring a chunk in
+// with whole-row loads, two chunks ahead in registers and two more in a ring of three LDS
+// buffers, behind a barrier that waits for LDS traffic only (a plain __syncthreads would wait for
+// the loads that are meant to stay in flight). Each chunk is read from memory once per 64 rows
+// instead of once per 16, and a wave's registers hold two small sets of pieces instead of a whole
+// chunk, so rows of every width get their chunks ahead of time.
+template <int KS, int CT>
+__global__ __launch_bounds__(256, (KS <= 10 ? 2 : 1)) void latent_attention_mfma_wg_kernel(
+    const bf16_t* __restrict__ qa, bf16_t* __restrict__ out, const bf16_t* __restrict__ kcache,
+    const int* __restrict__ block_table, int max_blocks, const int* __restrict__ cu_q,
+    const int* __restrict__ pos0, int H, int rank, int dc, float scale_log2, int window,
+    const bf16_t* __restrict__ gate, int gate_stride) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char la_lds[];
+  constexpr int NBUF = 3;
+  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+  const int c = lane % 16, g = lane / 16;
+  const int RS = dc + 8;
+  bf16_t* ring = reinterpret_cast<bf16_t*>(la_lds);       // [NBUF][32][RS]
+  const int b = blockIdx.y;
+  const int q0 = cu_q[b], qlen = cu_q[b + 1] - q0;
+  const int nrows = qlen * H;
+  // HALVES (rows too wide for one wave's registers): two tiles a workgroup, and two waves a tile,
+  // which form the same scores and sum one half of the coordinates each
+  constexpr bool HALVES = KS > 10;
+  constexpr int WG_ROWS = HALVES ? 32 : 64, CTP = HALVES ? CT / 2 : CT;
+  const int wg_row0 = blockIdx.x * WG_ROWS;
+  if (wg_row0 >= nrows) return;                           // the whole workgroup
+  const int p0 = pos0[b];
+  const int row0 = wg_row0 + 16 * (HALVES ? wave / 2 : wave);
+  const int qb0 = HALVES ? (wave % 2) * (CTP / 4) : 0;
+  const bool active = row0 < nrows;                       // a wave without rows still brings chunks in
+  int my_start[1], my_end[1];
+  bool ok[1];
+  LaFrag qf[1][KS];
+  {
+    const int row = row0 + c;
+    ok[0] = row < nrows;
+    const int qi = ok[0] ? row / H : 0;
+    my_end[0] = p0 + qi + 1;
+    my_start[0] = window > 0 ? (my_end[0] - window > 0 ? my_end[0] - window : 0) : 0;
+    const bf16_t* qrow = qa + ((size_t)q0 * H + (ok[0] ? row : 0)) * dc;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int d = 32 * ks + 8 * g;
+      qf[0][ks].q = (ok[0] && d < dc) ? *reinterpret_cast<const uint4*>(qrow + d) : uint4{0, 0, 0, 0};
+    }
+  }
+  // the wave's own keys and the workgroup's
+  const int w_last = (row0 + 15 < nrows - 1) ? row0 + 15 : nrows - 1;
+  const int w_end = active ? p0 + w_last / H + 1 : 0;
+  const int w_start = (active && window > 0 && p0 + row0 / H + 1 - window > 0) ? p0 + row0 / H + 1 - window : 0;
+  const int g_last = (wg_row0 + WG_ROWS - 1 < nrows - 1) ? wg_row0 + WG_ROWS - 1 : nrows - 1;
+  const int g_end = p0 + g_last / H + 1;
+  const int g_start = (window > 0 && p0 + wg_row0 / H + 1 - window > 0) ? p0 + wg_row0 / H + 1 - window : 0;
+  const int c0 = g_start / 32, n = (g_end + 31) / 32 - c0;
+  la_floatx4 O[1][CTP];
+#pragma unroll
+  for (int ct = 0; ct < CTP; ++ct) O[0][ct] = la_floatx4{0.f, 0.f, 0.f, 0.f};
+  float m[1] = {-INFINITY}, l[1] = {0.f};
+  const int* table = block_table + (size_t)b * max_blocks;
+  const int pieces = dc / 8, total = 32 * pieces;
+  constexpr int NP = (KS + 1) / 2;                        // pieces of a chunk a thread brings: 32 * 4 KS / 256
+  struct Set {
+    uint4 v[NP];
+  };
+  // loads without conditions (a piece that is not there reads the chunk's first): what is not
+  // there is decided when the pieces go to LDS, after the wait that is due then anyway
+  auto fetch = [&](Set& q, int i) {
+    const int key0 = (c0 + i) * 32;
+    const size_t page = (size_t)table[key0 / TA_PAGE];
+    const bf16_t* src = kcache + (page * TA_PAGE + key0 % TA_PAGE) * (size_t)dc;
+#pragma unroll
+    for (int u = 0; u < NP; ++u) {
+      const int idx = tid + 256 * u;
+      const int k = idx / pieces, pc = idx - k * pieces;
+      q.v[u] = *reinterpret_cast<const uint4*>(idx < total ? src + (size_t)k * dc + pc * 8 : src);
+    }
+  };
+  auto stash = [&](const Set& q, int i) {
+    const int key0 = (c0 + i) * 32;
+    bf16_t* Ks = ring + (size_t)(i % NBUF) * 32 * RS;
+#pragma unroll
+    for (int u = 0; u < NP; ++u) {
+      const int idx = tid + 256 * u;
+      const int k = idx / pieces, pc = idx - k * pieces;
+      if (idx < total)                                      // keys not written yet are stored as zero
+        *reinterpret_cast<uint4*>(Ks + k * RS + pc * 8) = key0 + k < g_end ? q.v[u] : uint4{0, 0, 0, 0};
+    }
+  };
+  auto multiply = [&](int i) {
+    const int key0 = (c0 + i) * 32;
+    if (!active || key0 + 32 <= w_start || key0 >= w_end) return;      // none of the wave's rows sees this chunk
+    la_chunk<KS, CTP, 1>(ring + (size_t)(i % NBUF) * 32 * RS, RS, dc, rank, key0, c, g, qf, ok, my_start, my_end,
+                         scale_log2, m, l, O, qb0);
+  };
+  auto lds_barrier = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+  Set sa, sb;
+  fetch(sa, 0);
+  if (n > 1) fetch(sb, 1);
+  stash(sa, 0);
+  if (n > 1) stash(sb, 1);
+  if (n > 2) fetch(sa, 2);
+  if (n > 3) fetch(sb, 3);
+  lds_barrier();
+  // chunk i is multiplied from buffer i % 3 while chunk i + 1 waits in the next buffer; the pieces
+  // of chunk i + 2 then leave their set for the third buffer and the set asks for chunk i + 4
+  for (int i = 0; i < n; i += 2) {
+    multiply(i);
+    if (i + 2 < n) {
+      stash(sa, i + 2);
+      if (i + 4 < n) fetch(sa, i + 4);
+    }
+    lds_barrier();
+    if (i + 1 >= n) break;
+    multiply(i + 1);
+    if (i + 3 < n) {
+      stash(sb, i + 3);
+      if (i + 5 < n) fetch(sb, i + 5);
+    }
+    lds_barrier();
+  }
+  if (!active || !ok[0]) return;
+  const int row = row0 + c;
+  float f = l[0] > 0.f ? 1.0f / l[0] : 0.f;
+  if (gate) {
+    const float gv = to_f32(gate[(size_t)(q0 + row / H) * gate_stride + row % H]);
+    f *= 1.0f / (1.0f + expf(-gv));
+  }
+  bf16_t* o = out + ((size_t)q0 * H + row) * rank;
+#pragma unroll
+  for (int ct = 0; ct < CTP; ++ct)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int coord = 64 * (qb0 + ct / 4) + 16 * g + 4 * j + (ct % 4);
+      if (coord < rank) o[coord] = from_f32<bf16_t>(O[0][ct][j] * f);
+    }
+}
+
+template <int KS, int CT>
+static int latent_mfma_wg_run(hipStream_t stream, dim3 g, size_t lds, const void* qa, void* out, const void* kcache,
+                              const int* block_table, int max_blocks, const int* cu_q, const int* pos0, int H,
+                              int rank, int dc, float scale_log2, int window, const void* gate, int gate_stride) {
+  auto kern = latent_attention_mfma_wg_kernel<KS, CT>;
+  static size_t allowed = 64 * 1024;                    // per instantiation: asked for once, not at every launch
+  if (lds > allowed) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return ta_fail("ta_latent_attention: %zu bytes of LDS refused (%s)", lds, hipGetErrorString(e));
+    allowed = lds;
+  }
+  kern<<<g, 256, lds, stream>>>((const bf16_t*)qa, (bf16_t*)out, (const bf16_t*)kcache, block_table, max_blocks,
+                                cu_q, pos0, H, rank, dc, scale_log2, window, (const bf16_t*)gate, gate_stride);
+  return 0;
 }
 
 // One wave per row: the shares of a row's keys are put together.
@@ -649,6 +815,22 @@ extern "C" int ta_latent_attention(hipStream_t stream, int dtype, const void* qa
   const int rows = dtype == TA_BF16 ? ta_latent_mfma_rows(rank, dc, max_qlen, H) : 0;
   if (rows > 0) {
     TA_REQUIRE(splits >= 1 && splits <= 65535 && (splits == 1 || scratch != nullptr), "ta_latent_attention: %d shares without scratch", splits);
+    if (splits == 1 && (long long)max_qlen * H >= 64) {   // many rows: workgroups of four tiles share their chunks
+      const int wg_rows = (dc <= 320 && rank <= 256) ? 64 : 32;      // wide rows: two waves a tile, see the kernel
+      const long long wgs = ((long long)max_qlen * H + wg_rows - 1) / wg_rows;
+      TA_REQUIRE(wgs <= 2147483647ll, "ta_latent_attention: too many rows");
+      dim3 gw((unsigned)wgs, batch);
+      const size_t ldw = (size_t)3 * 32 * (dc + 8) * sizeof(bf16_t);
+      const float sl2w = scale * 1.4426950408889634f;
+      int rcw;
+#define LA_WG(KS, CT) latent_mfma_wg_run<KS, CT>(stream, gw, ldw, qa, out, kcache, block_table, max_blocks, cu_q, pos0, H, rank, dc, sl2w, window, gate, gate_stride)
+      if (dc <= 192 && rank <= 128) rcw = LA_WG(6, 8);
+      else if (dc <= 320 && rank <= 256) rcw = LA_WG(10, 16);
+      else rcw = LA_WG(18, 32);
+#undef LA_WG
+      if (rcw) return rcw;
+      return ta_check_launch("ta_latent_attention");
+    }
     const long long tiles = ((long long)max_qlen * H + rows - 1) / rows;
     TA_REQUIRE(tiles <= 2147483647ll, "ta_latent_attention: too many rows");
     const bool halves = !(dc <= 320 && rank <= 256);      // two waves a tile: see the kernel
