@@ -1412,11 +1412,14 @@ def latent_row_width(rank: int, rot: int, dtype: torch.dtype) -> int:
 def latent_key_shares(batch: int, max_qlen: int, heads: int, rank: int, width: int, max_kv_len: int,
                       window: Optional[int]) -> int:
     """Waves that share a row's keys in ``latent_attention`` on the matrix cores: one when the
-    step's rows alone give the CUs enough waves, else enough to reach about two waves per SIMD
-    while a share keeps at least two chunks of 32 keys. A function of the step's shape only."""
+    step's rows alone give the CUs enough work (then the kernel whose workgroups share their
+    chunks runs), else enough to reach about two waves per SIMD while a share keeps at least
+    two chunks of 32 keys. A function of the step's shape only."""
     rows = int(library().ta_latent_mfma_rows(c_int(rank), c_int(width), c_int(max_qlen), c_int(heads)))
     if rows == 0:
         return 1
+    if max_qlen * heads >= 64 and batch * -(-max_qlen * heads // 64) >= 128:
+        return 1        # enough workgroups of four tiles that share their chunks (the kernel for many rows)
     waves = batch * -(-max_qlen * heads // rows)
     keys = max_kv_len if not window else min(max_kv_len, window + max_qlen)
     chunks = keys // 32 + 2
