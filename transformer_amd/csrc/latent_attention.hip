@@ -15,7 +15,10 @@
 //   latent_query_rot : the rotated part of every head's query, rotated, into the last `rot`
 //                      coordinates of the wide query rows
 //   latent_attention : causal (windowed) softmax attention of the wide queries over the
-//                      cached rows, float32 on the vector ALU, an output gate per (token, head)
+//                      cached rows with an output gate per (token, head): float32 on the
+//                      vector ALU; for bfloat16 rows on the matrix cores, with a workgroup's
+//                      waves sharing their chunks of keys in steps of many rows and a row's
+//                      keys dealt to several waves in steps of few
 //
 // Rotation: coordinates (2i, 2i + 1), i < dims / 2, of a rotated part turn by the token's
 // angle i; angles come as (cos, sin) float32 [nt, dims / 2, 2]. Everything between loads and
@@ -299,8 +302,8 @@ static int latent_attention_run(hipStream_t stream, dim3 g, size_t lds, const vo
 }
 
 // ------------------------------------------------------------------ the same on the matrix cores (bfloat16)
-// A wave owns RT tiles of 16 rows and a share of their keys; a workgroup is four such waves that
-// share nothing (no barrier between them). Keys come in chunks of 32 aligned to absolute
+// Steps of few rows: a wave owns RT tiles of 16 rows and a share of their keys; a workgroup is four
+// such waves that share nothing (no barrier between them). Keys come in chunks of 32 aligned to absolute
 // positions: the wave copies a chunk's rows into its own piece of LDS, forms S^T = K Q^T on
 // v_mfma_f32_16x16x32_bf16 (a lane then holds 4 keys x 2 tiles of ONE row: the softmax stays in
 // the lane but for two shuffles), and O^T += C^T P^T with the latent's coordinates gathered
